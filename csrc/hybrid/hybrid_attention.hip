@@ -2,8 +2,10 @@
 // per-head score multiplier, for any head sizes up to 256 (fp32 FMA form; bf16 or fp32 tensors).
 //
 //   K cache [num_blocks, G, BS, Dk], V cache [num_blocks, G, BS, Dv], q [T, H, Dk], out [T, H * Dv]
-//   score(i, j) = q_i . k_j * scale * temp[h], j <= position(i)
+//   score(i, j) = q_i . k_j * scale * temp[h] - slopes[h] * (i - j), j <= position(i),
+//                 and i - j < window when a window is given (tiles wholly ahead of it are skipped)
 //   weight_j   = exp(s_j) / (sink + sum_j exp(s_j))        (sink: a key of score 0 without a value)
+//   out       *= sigmoid(gate[row, h * Dv + col])          when a gate is given
 //
 // One workgroup of 4 waves = one work item (sequence, first row) x one key/value head x one key
 // range: up to 32 (row, head) pairs, 8 per wave, that all read the same keys and values. The keys
@@ -33,7 +35,8 @@ __global__ void __launch_bounds__(256) gqa_attention_kernel(
     const int* __restrict__ block_tables, const int* __restrict__ cu_q, const int* __restrict__ start_pos,
     const int* __restrict__ tiles, const float* __restrict__ temp, float* __restrict__ part_o,
     float* __restrict__ part_ml, int H, int G, int Dk, int Dv, int BS, int max_blocks, int R, int KT, int hchunks,
-    float scale, float sink) {
+    float scale, float sink, int window, const float* __restrict__ slopes, const T* __restrict__ gate,
+    int gate_stride) {
   extern __shared__ float lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int seq = tiles[2 * blockIdx.x], row0 = tiles[2 * blockIdx.x + 1];
@@ -44,11 +47,13 @@ __global__ void __launch_bounds__(256) gqa_attention_kernel(
   const int P = nrows * nh;
   const int pos0 = start_pos[seq] + (row0 - cu_q[seq]);           // position of the tile's first row
   const int kend = pos0 + nrows;                                  // keys 0 .. kend - 1 are visible to the tile
-  // this workgroup's key range (whole tiles of KT keys)
+  // this workgroup's key range (whole tiles of KT keys, counted from key 0; with a window the
+  // tiles that end before the first row's oldest visible key are left out: every weight in them is 0)
   const int S = gridDim.z;
   const int ntile = (kend + KT - 1) / KT;
-  const int per = (ntile + S - 1) / S;
-  const int t_lo = blockIdx.z * per, t_hi = min(ntile, t_lo + per);
+  const int t0 = window > 0 ? max(0, pos0 - window + 1) / KT : 0;
+  const int per = (ntile - t0 + S - 1) / S;
+  const int t_lo = t0 + blockIdx.z * per, t_hi = min(ntile, t_lo + per);
 
   float* qs = lds;                              // [kWaves * kPW][Dk]
   float* ks = qs + kWaves * kPW * Dk;           // [KT][Dk + 1]
@@ -61,7 +66,7 @@ __global__ void __launch_bounds__(256) gqa_attention_kernel(
     const int r = p / nh, h = g * group + h_lo + (p - r * nh);
     qs[i] = DT<T>::load(q + ((size_t)(row0 + r) * H + h) * Dk + d);
   }
-  float m[kPW], l[kPW], hs[kPW], o[kPW][DVL];
+  float m[kPW], l[kPW], hs[kPW], sl[kPW], o[kPW][DVL];
   int qpos[kPW];
 #pragma unroll
   for (int i = 0; i < kPW; ++i) {
@@ -71,6 +76,7 @@ __global__ void __launch_bounds__(256) gqa_attention_kernel(
     const int r = p / nh, h = g * group + h_lo + (p - r * nh);
     qpos[i] = p < P ? pos0 + r : -1;
     hs[i] = p < P ? scale * (temp ? temp[h] : 1.0f) : 0.f;
+    sl[i] = p < P && slopes ? slopes[h] : 0.f;
 #pragma unroll
     for (int c = 0; c < DVL; ++c) o[i][c] = 0.f;
   }
@@ -108,8 +114,9 @@ __global__ void __launch_bounds__(256) gqa_attention_kernel(
     float alpha[kPW];
 #pragma unroll
     for (int i = 0; i < kPW; ++i) {
-      const bool ok = lane < KT && kb + lane <= qpos[i];
-      const float sc = ok ? s[i] * hs[i] : kNeg;
+      const int dist = qpos[i] - (kb + lane);
+      const bool ok = lane < KT && dist >= 0 && (window <= 0 || dist < window);
+      const float sc = ok ? s[i] * hs[i] - sl[i] * (float)dist : kNeg;
       const float mn = fmaxf(m[i], rt::wave_max(sc));
       const float pe = ok ? __expf(sc - mn) : 0.f;
       alpha[i] = __expf(m[i] - mn);
@@ -149,7 +156,11 @@ __global__ void __launch_bounds__(256) gqa_attention_kernel(
 #pragma unroll
       for (int c = 0; c < DVL; ++c) {
         const int col = lane + 64 * c;
-        if (col < Dv) DT<T>::store(out + rh * Dv + col, o[i][c] * inv);
+        if (col < Dv) {
+          float v = o[i][c] * inv;
+          if (gate) v *= 1.0f / (1.0f + __expf(-DT<T>::load(gate + (size_t)(row0 + r) * gate_stride + h * Dv + col)));
+          DT<T>::store(out + rh * Dv + col, v);
+        }
       }
     } else {
       float* po = part_o + (rh * S + blockIdx.z) * Dv;
@@ -169,7 +180,8 @@ __global__ void __launch_bounds__(256) gqa_attention_kernel(
 // one wave per (row, head): merge the S partials, add the sink once
 template <typename T>
 __global__ void __launch_bounds__(64) gqa_combine_kernel(T* __restrict__ out, const float* __restrict__ part_o,
-                                                         const float* __restrict__ part_ml, int S, int Dv, float sink) {
+                                                         const float* __restrict__ part_ml, int S, int Dv, float sink,
+                                                         int H, const T* __restrict__ gate, int gate_stride) {
   const size_t rh = blockIdx.x;
   const int lane = threadIdx.x;
   float M = kNeg;
@@ -180,7 +192,9 @@ __global__ void __launch_bounds__(64) gqa_combine_kernel(T* __restrict__ out, co
   for (int col = lane; col < Dv; col += 64) {
     float acc = 0.f;
     for (int s = 0; s < S; ++s) acc += part_o[(rh * S + s) * Dv + col] * __expf(part_ml[(rh * S + s) * 2] - M);
-    DT<T>::store(out + rh * Dv + col, acc * inv);
+    float v = acc * inv;
+    if (gate) v *= 1.0f / (1.0f + __expf(-DT<T>::load(gate + (rh / H) * gate_stride + (rh % H) * Dv + col)));
+    DT<T>::store(out + rh * Dv + col, v);
   }
 }
 
@@ -200,7 +214,8 @@ int gqa_key_tile(int Dk, int Dv) {
 int launch_gqa_attention(void* out, const void* q, const void* kc, const void* vc, const int* block_tables,
                          const int* cu_q, const int* start_pos, const int* tiles, int n_tiles, const float* temp,
                          float* part_o, float* part_ml, int T, int H, int G, int Dk, int Dv, int BS, int max_blocks,
-                         int rows, int num_splits, float scale, float sink, bool bf, hipStream_t stream) {
+                         int rows, int num_splits, float scale, float sink, int window, const float* slopes,
+                         const void* gate, int gate_stride, bool bf, hipStream_t stream) {
   if (n_tiles <= 0 || T <= 0) return 0;
   const int KT = gqa_key_tile(Dk, Dv);
   if (KT == 0 || Dv > 256 || Dk > 256 || H % G) return -1;
@@ -224,7 +239,7 @@ int launch_gqa_attention(void* out, const void* q, const void* kc, const void* v
       return -3;                                                                                                     \
     kern<<<grid, 256, shm, stream>>>((TT*)out, (const TT*)q, (const TT*)kc, (const TT*)vc, block_tables, cu_q,      \
                                      start_pos, tiles, temp, part_o, part_ml, H, G, Dk, Dv, BS, max_blocks, rows,   \
-                                     KT, hchunks, scale, sink);                                                      \
+                                     KT, hchunks, scale, sink, window, slopes, (const TT*)gate, gate_stride);        \
   } while (0)
   if (bf) {
     if (dvl == 1) RT_GQA(uint16_t, 1); else if (dvl == 2) RT_GQA(uint16_t, 2); else RT_GQA(uint16_t, 4);
@@ -234,8 +249,10 @@ int launch_gqa_attention(void* out, const void* q, const void* kc, const void* v
 #undef RT_GQA
 #undef RT_GQA2
   if (num_splits > 1) {
-    if (bf) gqa_combine_kernel<uint16_t><<<T * H, 64, 0, stream>>>((uint16_t*)out, part_o, part_ml, num_splits, Dv, sink);
-    else gqa_combine_kernel<float><<<T * H, 64, 0, stream>>>((float*)out, part_o, part_ml, num_splits, Dv, sink);
+    if (bf) gqa_combine_kernel<uint16_t><<<T * H, 64, 0, stream>>>((uint16_t*)out, part_o, part_ml, num_splits, Dv, sink, H,
+                                                                   (const uint16_t*)gate, gate_stride);
+    else gqa_combine_kernel<float><<<T * H, 64, 0, stream>>>((float*)out, part_o, part_ml, num_splits, Dv, sink, H,
+                                                             (const float*)gate, gate_stride);
   }
   return 0;
 }

@@ -1,0 +1,208 @@
+// H9 .. H12: feed-forward kernels. All math fp32; tensors bf16 (uint16_t storage) or fp32.
+//
+//   xielu            z = a + bias; z > 0: ap z^2 + z / 2; else an (e^z - 1 - z) + z / 2
+//   silu_glu         gu = (gate | up) [T, 2F] -> silu(gate) * up
+//   topk_softmax     per row of fp32 router logits: the `top` largest (lower index wins a tie) and
+//                    the softmax over those alone
+//   moe_rows         a few rows through their experts, two launches (the decode-step form of a
+//                    mixture of gated experts, no host round trip so a graph can hold it):
+//                    hid[t, k, :] = silu(Wg[e] h_t) * (Wu[e] h_t),  e = idx[t, k]
+//                    out[t, :]    = sum_k wt[t, k] * Wd[e] hid[t, k, :]
+//                    One wave per output entry walks a weight row in 16-byte loads against the
+//                    input row staged in LDS as fp32; a row's result does not depend on the others.
+#include "../common.h"
+
+namespace {
+
+using rt::DT;
+
+RT_DEVICE float sigm(float v) { return 1.0f / (1.0f + expf(-v)); }
+
+template <typename T>
+__global__ void __launch_bounds__(256) xielu_kernel(T* __restrict__ out, const T* __restrict__ a,
+                                                    const float* __restrict__ bias, int64_t n, int F, float ap, float an) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float z = DT<T>::load(a + i) + (bias ? bias[i % F] : 0.f);
+  DT<T>::store(out + i, z > 0.f ? ap * z * z + 0.5f * z : an * (expm1f(z) - z) + 0.5f * z);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) silu_glu_kernel(T* __restrict__ out, const T* __restrict__ gu, int64_t rows, int F) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= rows * F) return;
+  const int64_t r = i / F;
+  const int c = (int)(i - r * F);
+  const float g = DT<T>::load(gu + r * 2 * F + c);
+  DT<T>::store(out + i, g * sigm(g) * DT<T>::load(gu + r * 2 * F + F + c));
+}
+
+constexpr int kTopPerLane = 8;      // experts per lane: up to 512 experts
+
+__global__ void __launch_bounds__(64) topk_softmax_kernel(int* __restrict__ idx, float* __restrict__ wt,
+                                                          const float* __restrict__ logits, int E, int top) {
+  const int t = blockIdx.x, lane = threadIdx.x;
+  float v[kTopPerLane];
+#pragma unroll
+  for (int q = 0; q < kTopPerLane; ++q) {
+    const int e = lane + 64 * q;
+    v[q] = e < E ? logits[(size_t)t * E + e] : -INFINITY;
+  }
+  float mine = 0.f, first = 0.f;      // lane k keeps the k-th chosen logit
+  int mine_e = 0;
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY;
+    int be = 1 << 30;
+#pragma unroll
+    for (int q = 0; q < kTopPerLane; ++q)
+      if (v[q] > best) {
+        best = v[q];
+        be = lane + 64 * q;
+      }
+    const float top_v = rt::wave_max(best);
+    int cand = best == top_v ? be : 1 << 30;
+    for (int o = 32; o; o >>= 1) cand = min(cand, __shfl_xor(cand, o));
+#pragma unroll
+    for (int q = 0; q < kTopPerLane; ++q)
+      if (lane + 64 * q == cand) v[q] = -INFINITY;
+    if (k == 0) first = top_v;
+    if (lane == k) {
+      mine = top_v;
+      mine_e = min(cand, E - 1);     // (only all-NaN logits leave no candidate)
+    }
+  }
+  const float e = lane < top ? expf(mine - first) : 0.f;
+  const float sum = rt::wave_sum(e);
+  if (lane < top) {
+    idx[(size_t)t * top + lane] = mine_e;
+    wt[(size_t)t * top + lane] = e / sum;
+  }
+}
+
+// sum over n entries of w[i] * x[i] for the whole wave; x fp32 in LDS, w a weight row in memory
+template <typename T>
+RT_DEVICE float wave_dot(const T* __restrict__ w, const float* __restrict__ x, int n, int lane);
+
+template <>
+RT_DEVICE float wave_dot<uint16_t>(const uint16_t* __restrict__ w, const float* __restrict__ x, int n, int lane) {
+  float acc = 0.f;
+  if ((n & 7) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0) {
+    for (int c = lane * 8; c < n; c += 512) {
+      const rt::short8 p = *reinterpret_cast<const rt::short8*>(w + c);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) acc += rt::bf2f((uint16_t)p[q]) * x[c + q];
+    }
+  } else {
+    for (int c = lane; c < n; c += 64) acc += rt::bf2f(w[c]) * x[c];
+  }
+  return rt::wave_sum(acc);
+}
+
+template <>
+RT_DEVICE float wave_dot<float>(const float* __restrict__ w, const float* __restrict__ x, int n, int lane) {
+  float acc = 0.f;
+  if ((n & 3) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0) {
+    for (int c = lane * 4; c < n; c += 256) {
+      const float4 p = *reinterpret_cast<const float4*>(w + c);
+      acc += p.x * x[c] + p.y * x[c + 1] + p.z * x[c + 2] + p.w * x[c + 3];
+    }
+  } else {
+    for (int c = lane; c < n; c += 64) acc += w[c] * x[c];
+  }
+  return rt::wave_sum(acc);
+}
+
+constexpr int kMoeWaves = 4;
+
+// grid (T * top, blocks over F); wgu [E, 2F, W] = (gate | up) rows of every expert
+template <typename T>
+__global__ void __launch_bounds__(64 * kMoeWaves) moe_gate_up_kernel(float* __restrict__ hid, const T* __restrict__ h,
+                                                                     const T* __restrict__ wgu,
+                                                                     const int* __restrict__ idx, int W, int F, int top,
+                                                                     int per_block) {
+  extern __shared__ float xs[];
+  const int pair = blockIdx.x, t = pair / top;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) xs[c] = DT<T>::load(h + (size_t)t * W + c);
+  __syncthreads();
+  const T* we = wgu + (size_t)idx[pair] * 2 * F * W;
+  const int f0 = blockIdx.y * per_block, f1 = min(F, f0 + per_block);
+  for (int f = f0 + wave; f < f1; f += kMoeWaves) {
+    const float g = wave_dot<T>(we + (size_t)f * W, xs, W, lane);
+    const float u = wave_dot<T>(we + (size_t)(F + f) * W, xs, W, lane);
+    if (lane == 0) hid[(size_t)pair * F + f] = g * sigm(g) * u;
+  }
+}
+
+// grid (T, blocks over W); wd [E, W, F]
+template <typename T>
+__global__ void __launch_bounds__(64 * kMoeWaves) moe_down_kernel(T* __restrict__ out, const float* __restrict__ hid,
+                                                                  const T* __restrict__ wd, const int* __restrict__ idx,
+                                                                  const float* __restrict__ wt, int W, int F, int top,
+                                                                  int per_block) {
+  extern __shared__ float xs[];       // [top][F]
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int c = threadIdx.x; c < top * F; c += blockDim.x) xs[c] = hid[(size_t)t * top * F + c];
+  __syncthreads();
+  const int c0 = blockIdx.y * per_block, c1 = min(W, c0 + per_block);
+  for (int c = c0 + wave; c < c1; c += kMoeWaves) {
+    float acc = 0.f;
+    for (int k = 0; k < top; ++k)
+      acc += wt[(size_t)t * top + k] *
+             wave_dot<T>(wd + ((size_t)idx[(size_t)t * top + k] * W + c) * F, xs + (size_t)k * F, F, lane);
+    if (lane == 0) DT<T>::store(out + (size_t)t * W + c, acc);
+  }
+}
+
+}  // namespace
+
+void launch_xielu(void* out, const void* a, const float* bias, int64_t rows, int F, float ap, float an, bool bf,
+                  hipStream_t stream) {
+  const int64_t n = rows * F;
+  if (n <= 0) return;
+  const int blocks = (int)((n + 255) / 256);
+  if (bf) xielu_kernel<uint16_t><<<blocks, 256, 0, stream>>>((uint16_t*)out, (const uint16_t*)a, bias, n, F, ap, an);
+  else xielu_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)a, bias, n, F, ap, an);
+}
+
+void launch_silu_glu(void* out, const void* gu, int64_t rows, int F, bool bf, hipStream_t stream) {
+  const int64_t n = rows * F;
+  if (n <= 0) return;
+  const int blocks = (int)((n + 255) / 256);
+  if (bf) silu_glu_kernel<uint16_t><<<blocks, 256, 0, stream>>>((uint16_t*)out, (const uint16_t*)gu, rows, F);
+  else silu_glu_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)gu, rows, F);
+}
+
+int launch_topk_softmax(int* idx, float* wt, const float* logits, int T, int E, int top, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (E > 64 * kTopPerLane || top > 64 || top < 1 || top > E) return -1;
+  topk_softmax_kernel<<<T, 64, 0, stream>>>(idx, wt, logits, E, top);
+  return 0;
+}
+
+int launch_moe_rows(void* out, float* hid, const void* h, const void* wgu, const void* wd, const int* idx,
+                    const float* wt, int T, int W, int F, int top, bool bf, hipStream_t stream) {
+  if (T <= 0) return 0;
+  const size_t shm1 = sizeof(float) * (size_t)W, shm2 = sizeof(float) * (size_t)top * F;
+  if (shm1 > 150 * 1024 || shm2 > 150 * 1024) return -1;
+  // about 16 output entries per wave: enough workgroups to fill the chip from a handful of rows
+  const int pb = 16 * kMoeWaves;
+  const dim3 g1(T * top, (F + pb - 1) / pb), g2(T, (W + pb - 1) / pb);
+#define RT_MOE(TT)                                                                                                     \
+  do {                                                                                                                 \
+    auto k1 = moe_gate_up_kernel<TT>;                                                                                  \
+    auto k2 = moe_down_kernel<TT>;                                                                                     \
+    if (shm1 > 48 * 1024 &&                                                                                            \
+        hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm1) != hipSuccess)     \
+      return -2;                                                                                                       \
+    if (shm2 > 48 * 1024 &&                                                                                            \
+        hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm2) != hipSuccess)     \
+      return -2;                                                                                                       \
+    k1<<<g1, 64 * kMoeWaves, shm1, stream>>>(hid, (const TT*)h, (const TT*)wgu, idx, W, F, top, pb);                   \
+    k2<<<g2, 64 * kMoeWaves, shm2, stream>>>((TT*)out, hid, (const TT*)wd, idx, wt, W, F, top, pb);                    \
+  } while (0)
+  if (bf) RT_MOE(uint16_t); else RT_MOE(float);
+#undef RT_MOE
+  return 0;
+}

@@ -3,11 +3,15 @@
 // per row (H4: per sequence and 256 channels); rows are read twice (the second read hits L1 / L2),
 // never staged in LDS, so any row width runs.
 //
-//   shift_norm        xs = x + y ; h = xs / rms(xs) * w ; out = h + (h_prev - h) * mu
+//   shift_norm        xs = x + y ; h = xs / rms(xs) * w ; out_m = h + (h_prev - h) * mu_m, m < n_mix
 //                     h_prev: the row above inside a span, the sequence's state at a span's first
 //                     row, zero at position 0; optionally stores h as the new state (decode step)
+//                     (the norms of this file work on `groups` equal parts of a row, each divided
+//                     by its own root mean square: blockIdx.y is the part)
 //   shift_state       state[slot] = normed last row of every span
-//   qk_prep           rotary pairs (2i, 2i + 1), per-head x / rms(x); keys, values -> paged cache
+//   qk_prep           rotary pairs (2i, 2i + 1), per-head x / rms(x) (* a weight per channel; queries
+//                     * 1 + coef ln(floor((p + 1) / every) + 1)); values optionally / rms(v);
+//                     keys, values -> paged cache
 //   mingru_scan       z = sigmoid(.), c = u + 1/2 | sigmoid(u); S = (1 - z) S + z c; out = S silu(g)
 //   dual_norm_add     x += (a / rms(a) * wa + b / rms(b) * wb) / 2
 //   add_norm          x += y ; out = x / rms(x) * w
@@ -42,21 +46,24 @@ __global__ void __launch_bounds__(1024) shift_norm_kernel(
     OT* __restrict__ out, float* __restrict__ xs, const float* __restrict__ x, const YT* __restrict__ y,
     const float* __restrict__ w, const float* __restrict__ mu, float* __restrict__ state,
     const int* __restrict__ row_seq, const int64_t* __restrict__ positions, const int* __restrict__ start_pos,
-    const int* __restrict__ slots, int W, float eps, int store_state) {
+    const int* __restrict__ slots, int W, int Wg, int n_mix, float eps, int store_state) {
   __shared__ float scratch[32];
   const int t = blockIdx.x;
+  const int c0 = blockIdx.y * Wg;                        // this workgroup's part of the row
+  const size_t T = gridDim.x;
   const int s = row_seq[t];
   const int64_t pos = positions[t];
   const bool first = pos == (int64_t)start_pos[s];      // first row of its span in this launch
-  const float* xr = x + (size_t)t * W;
-  const YT* yr = y ? y + (size_t)t * W : nullptr;
+  const float* xr = x + (size_t)t * W + c0;
+  const YT* yr = y ? y + (size_t)t * W + c0 : nullptr;
   const float* xp = xr - W;                              // only read when !first (then t > 0)
   const YT* yp = yr ? yr - W : nullptr;
-  float* st = state + (size_t)slots[s] * W;
+  float* st = state + (size_t)slots[s] * W + c0;
+  const float* wg = w + c0;
   float ss = 0.f, sp = 0.f;
   float cv[kKeep], cu[kKeep];     // this row's and the row above's first entries per lane
   int i = 0;
-  for (int c = threadIdx.x; c < W; c += blockDim.x, ++i) {
+  for (int c = threadIdx.x; c < Wg; c += blockDim.x, ++i) {
     const float v = xr[c] + (yr ? DT<YT>::load(yr + c) : 0.f);
     ss += v * v;
     float u = 0.f;
@@ -72,9 +79,9 @@ __global__ void __launch_bounds__(1024) shift_norm_kernel(
       }
   }
   block_sum2(ss, sp, scratch);
-  const float kc = inv_rms(ss, W, eps), kp = inv_rms(sp, W, eps);
+  const float kc = inv_rms(ss, Wg, eps), kp = inv_rms(sp, Wg, eps);
   i = 0;
-  for (int c = threadIdx.x; c < W; c += blockDim.x, ++i) {
+  for (int c = threadIdx.x; c < Wg; c += blockDim.x, ++i) {
     float v = 0.f, u = 0.f;
     if (i < kKeep) {
 #pragma unroll
@@ -87,29 +94,31 @@ __global__ void __launch_bounds__(1024) shift_norm_kernel(
       v = xr[c] + (yr ? DT<YT>::load(yr + c) : 0.f);
       if (!first) u = xp[c] + (yp ? DT<YT>::load(yp + c) : 0.f);
     }
-    const float h = v * kc * w[c];
+    const float h = v * kc * wg[c];
     float hp;
-    if (!first) hp = u * kp * w[c];
+    if (!first) hp = u * kp * wg[c];
     else hp = pos > 0 ? st[c] : 0.f;
-    DT<OT>::store(out + (size_t)t * W + c, h + (hp - h) * mu[c]);
-    if (yr) xs[(size_t)t * W + c] = v;
+    for (int m = 0; m < n_mix; ++m)
+      DT<OT>::store(out + ((size_t)m * T + t) * W + c0 + c, h + (hp - h) * mu[(size_t)m * W + c0 + c]);
+    if (yr) xs[(size_t)t * W + c0 + c] = v;
     if (store_state) st[c] = h;
   }
 }
 
 __global__ void __launch_bounds__(1024) shift_state_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                            float* __restrict__ state, const int* __restrict__ cu_q,
-                                                           const int* __restrict__ slots, int W, float eps) {
+                                                           const int* __restrict__ slots, int W, int Wg, float eps) {
   __shared__ float scratch[16];
   const int s = blockIdx.x;
+  const int c0 = blockIdx.y * Wg;
   const int n = cu_q[s + 1] - cu_q[s];
   if (n <= 0) return;
-  const float* xr = x + (size_t)(cu_q[s + 1] - 1) * W;
+  const float* xr = x + (size_t)(cu_q[s + 1] - 1) * W + c0;
   float ss = 0.f;
-  for (int c = threadIdx.x; c < W; c += blockDim.x) ss += xr[c] * xr[c];
-  const float k = inv_rms(rt::block_sum(ss, scratch), W, eps);
-  float* st = state + (size_t)slots[s] * W;
-  for (int c = threadIdx.x; c < W; c += blockDim.x) st[c] = xr[c] * k * w[c];
+  for (int c = threadIdx.x; c < Wg; c += blockDim.x) ss += xr[c] * xr[c];
+  const float k = inv_rms(rt::block_sum(ss, scratch), Wg, eps);
+  float* st = state + (size_t)slots[s] * W + c0;
+  for (int c = threadIdx.x; c < Wg; c += blockDim.x) st[c] = xr[c] * k * w[c0 + c];
 }
 
 // One wave per head unit: units 0 .. H - 1 are query heads, H .. H + G - 1 key heads (each also
@@ -119,7 +128,8 @@ __global__ void __launch_bounds__(1024) qk_prep_kernel(
     T* __restrict__ q, const T* __restrict__ proj, int stride, int q_off, int k_off, int v_off, int v_from_k,
     const float* __restrict__ inv_freq, int rot_dims, float eps, const int64_t* __restrict__ positions,
     T* __restrict__ kc, T* __restrict__ vc, const int64_t* __restrict__ slot_mapping, int H, int G, int Dk, int Dv,
-    int BS, int layout, const float* __restrict__ q_scale) {
+    int BS, int layout, const float* __restrict__ q_scale, const float* __restrict__ q_w,
+    const float* __restrict__ k_w, int v_norm, float qt_coef, int qt_every) {
   __shared__ float cs_tab[256];      // (cos, sin) of the row's angles, once for all its heads
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const float pos = (float)positions[t];
@@ -157,6 +167,9 @@ __global__ void __launch_bounds__(1024) qk_prep_kernel(
     }
     float k = inv_rms(rt::wave_sum(ss), Dk, eps);
     if (is_q && q_scale) k *= q_scale[u];
+    // the query factor grows with the logarithm of the position, in steps of qt_every positions
+    if (is_q && qt_every > 0) k *= 1.0f + qt_coef * logf((float)((positions[t] + 1) / qt_every) + 1.0f);
+    const float* nw = is_q ? q_w : k_w;                  // a learned weight per channel, or none
     // layout 1: the matrix-core attention kernels' cache (keys chunk-major per block, rt::kc_elem;
     // values transposed [Dv][BS])
     T* dst = is_q ? q + ((size_t)t * H + u) * Dk
@@ -164,13 +177,22 @@ __global__ void __launch_bounds__(1024) qk_prep_kernel(
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int d = lane + 64 * j;
-      if (d < Dk) DT<T>::store(dst + ((!is_q && layout) ? rt::kc_elem(BS, off, d) : d), val[j] * k);
+      if (d < Dk) DT<T>::store(dst + ((!is_q && layout) ? rt::kc_elem(BS, off, d) : d), val[j] * k * (nw ? nw[d] : 1.0f));
     }
     if (!is_q) {
       const int g = u - H;
       const T* vs = v_from_k ? src : row + v_off + g * Dv;
       T* vd = vc + ((size_t)blk * G + g) * BS * Dv;
-      if (layout) for (int d = lane; d < Dv; d += 64) vd[(size_t)d * BS + off] = vs[d];
+      if (v_norm) {                                      // unit-RMS values, cached so
+        float sv = 0.f;
+        for (int d = lane; d < Dv; d += 64) {
+          const float a = DT<T>::load(vs + d);
+          sv += a * a;
+        }
+        const float kv = inv_rms(rt::wave_sum(sv), Dv, eps);
+        for (int d = lane; d < Dv; d += 64)
+          DT<T>::store(vd + (layout ? (size_t)d * BS + off : (size_t)off * Dv + d), DT<T>::load(vs + d) * kv);
+      } else if (layout) for (int d = lane; d < Dv; d += 64) vd[(size_t)d * BS + off] = vs[d];
       else for (int d = lane; d < Dv; d += 64) vd[(size_t)off * Dv + d] = vs[d];
     }
   }
@@ -282,23 +304,26 @@ __global__ void __launch_bounds__(1024) dual_norm_add_kernel(float* __restrict__
 template <typename OT, typename YT>
 __global__ void __launch_bounds__(1024) add_norm_kernel(OT* __restrict__ out, float* __restrict__ x,
                                                         const YT* __restrict__ y, const float* __restrict__ w, int W,
-                                                        float eps) {
+                                                        int Wg, float eps) {
   __shared__ float scratch[16];
-  float* xr = x + (size_t)blockIdx.x * W;
-  const YT* yr = y ? y + (size_t)blockIdx.x * W : nullptr;
+  const int c0 = blockIdx.y * Wg;                        // this workgroup's part of the row
+  float* xr = x + (size_t)blockIdx.x * W + c0;
+  const YT* yr = y ? y + (size_t)blockIdx.x * W + c0 : nullptr;
+  w += c0;
+  out += (size_t)blockIdx.x * W + c0;
   float ss = 0.f;
   float cv[kKeep];
   int i = 0;
-  for (int c = threadIdx.x; c < W; c += blockDim.x, ++i) {
+  for (int c = threadIdx.x; c < Wg; c += blockDim.x, ++i) {
     const float v = xr[c] + (yr ? DT<YT>::load(yr + c) : 0.f);
     ss += v * v;
 #pragma unroll
     for (int j = 0; j < kKeep; ++j)
       if (j == i) cv[j] = v;
   }
-  const float k = inv_rms(rt::block_sum(ss, scratch), W, eps);
+  const float k = inv_rms(rt::block_sum(ss, scratch), Wg, eps);
   i = 0;
-  for (int c = threadIdx.x; c < W; c += blockDim.x, ++i) {
+  for (int c = threadIdx.x; c < Wg; c += blockDim.x, ++i) {
     float v = 0.f;
     if (i < kKeep) {
 #pragma unroll
@@ -308,7 +333,7 @@ __global__ void __launch_bounds__(1024) add_norm_kernel(OT* __restrict__ out, fl
       v = xr[c] + (yr ? DT<YT>::load(yr + c) : 0.f);
     }
     if (yr) xr[c] = v;
-    DT<OT>::store(out + (size_t)blockIdx.x * W + c, v * k * w[c]);
+    DT<OT>::store(out + c, v * k * w[c]);
   }
 }
 
@@ -354,13 +379,15 @@ int row_threads(int W) {
 
 void launch_shift_norm(void* out, float* xs, const float* x, const void* y, const float* w, const float* mu,
                        float* state, const int* row_seq, const int64_t* positions, const int* start_pos,
-                       const int* slots, int T, int W, float eps, bool out_bf, bool y_bf, bool store_state,
-                       hipStream_t stream) {
+                       const int* slots, int T, int W, int groups, int n_mix, float eps, bool out_bf, bool y_bf,
+                       bool store_state, hipStream_t stream) {
   if (T <= 0) return;
-  const int th = row_threads(W);
-#define RT_SN(OT, YT)                                                                                              \
-  shift_norm_kernel<OT, YT><<<T, th, 0, stream>>>((OT*)out, xs, x, (const YT*)y, w, mu, state, row_seq, positions, \
-                                                  start_pos, slots, W, eps, store_state ? 1 : 0)
+  const int Wg = W / groups;
+  const int th = row_threads(Wg);
+  const dim3 grid(T, groups);
+#define RT_SN(OT, YT)                                                                                                 \
+  shift_norm_kernel<OT, YT><<<grid, th, 0, stream>>>((OT*)out, xs, x, (const YT*)y, w, mu, state, row_seq, positions, \
+                                                     start_pos, slots, W, Wg, n_mix, eps, store_state ? 1 : 0)
   if (out_bf) {
     if (y_bf) RT_SN(uint16_t, uint16_t); else RT_SN(uint16_t, float);
   } else {
@@ -370,26 +397,30 @@ void launch_shift_norm(void* out, float* xs, const float* x, const void* y, cons
 }
 
 void launch_shift_state(const float* x, const float* w, float* state, const int* cu_q, const int* slots, int S, int W,
-                        float eps, hipStream_t stream) {
+                        int groups, float eps, hipStream_t stream) {
   if (S <= 0) return;
-  shift_state_kernel<<<S, row_threads(W), 0, stream>>>(x, w, state, cu_q, slots, W, eps);
+  const int Wg = W / groups;
+  shift_state_kernel<<<dim3(S, groups), row_threads(Wg), 0, stream>>>(x, w, state, cu_q, slots, W, Wg, eps);
 }
 
 void launch_qk_prep(void* q, const void* proj, int stride, int q_off, int k_off, int v_off, bool v_from_k,
                     const float* inv_freq, int rot_dims, float eps, const int64_t* positions, void* kc, void* vc,
                     const int64_t* slot_mapping, int T, int H, int G, int Dk, int Dv, int BS, bool bf, int layout,
-                    const float* q_scale, hipStream_t stream) {
+                    const float* q_scale, const float* q_w, const float* k_w, bool v_norm, float qt_coef, int qt_every,
+                    hipStream_t stream) {
   if (T <= 0) return;
   // one wave per head unit, up to 16 waves a row: a decode step's few rows spread over whole workgroups
   const int th = T > 64 ? 256 : 64 * (H + G < 4 ? 4 : H + G > 16 ? 16 : H + G);
   if (bf)
     qk_prep_kernel<uint16_t><<<T, th, 0, stream>>>((uint16_t*)q, (const uint16_t*)proj, stride, q_off, k_off, v_off,
                                                     v_from_k, inv_freq, rot_dims, eps, positions, (uint16_t*)kc,
-                                                    (uint16_t*)vc, slot_mapping, H, G, Dk, Dv, BS, layout, q_scale);
+                                                    (uint16_t*)vc, slot_mapping, H, G, Dk, Dv, BS, layout, q_scale,
+                                                    q_w, k_w, v_norm ? 1 : 0, qt_coef, qt_every);
   else
     qk_prep_kernel<float><<<T, th, 0, stream>>>((float*)q, (const float*)proj, stride, q_off, k_off, v_off, v_from_k,
                                                  inv_freq, rot_dims, eps, positions, (float*)kc, (float*)vc,
-                                                 slot_mapping, H, G, Dk, Dv, BS, layout, q_scale);
+                                                 slot_mapping, H, G, Dk, Dv, BS, layout, q_scale, q_w, k_w,
+                                                 v_norm ? 1 : 0, qt_coef, qt_every);
 }
 
 void launch_mingru_scan(void* out, const void* proj, int stride, int z_off, int x_off, int g_off, int width,
@@ -440,11 +471,13 @@ void launch_dual_norm_add(float* x, const void* a, const float* wa, const void* 
     dual_norm_add_kernel<float><<<T, row_threads(W), 0, stream>>>(x, (const float*)a, wa, (const float*)b, wb, W, eps);
 }
 
-void launch_add_norm(void* out, float* x, const void* y, const float* w, int T, int W, float eps, bool out_bf,
-                     bool y_bf, hipStream_t stream) {
+void launch_add_norm(void* out, float* x, const void* y, const float* w, int T, int W, int groups, float eps,
+                     bool out_bf, bool y_bf, hipStream_t stream) {
   if (T <= 0) return;
-  const int th = row_threads(W);
-#define RT_AN(OT, YT) add_norm_kernel<OT, YT><<<T, th, 0, stream>>>((OT*)out, x, (const YT*)y, w, W, eps)
+  const int Wg = W / groups;
+  const int th = row_threads(Wg);
+  const dim3 grid(T, groups);
+#define RT_AN(OT, YT) add_norm_kernel<OT, YT><<<grid, th, 0, stream>>>((OT*)out, x, (const YT*)y, w, W, Wg, eps)
   if (out_bf) {
     if (y_bf) RT_AN(uint16_t, uint16_t); else RT_AN(uint16_t, float);
   } else {

@@ -300,30 +300,38 @@ class GroupedKVCache(StatefulPagedCache):
     matrix-core attention kernels instead: ``v[l]`` ``[num_blocks, kv_heads_l, vdim_l, block_size]``
     and each key block chunk-major (``ops/reference.py`` ``k_blocks``).
 
+    A run whose mixer has no attention gives ``None`` as its shape and has no pages (``k[l]`` and
+    ``v[l]`` are None): its memory per sequence is its state alone.
+
     States, fp32, one row per slot: ``shift[l]`` ``[n_slots, width]`` is the previous token's
-    normed mixer input (token shift); ``rec[l]`` ``[n_slots, rec_width_l]`` the state of the
-    layer's recurrence (None for a layer without one). A sequence at position 0 never reads its
-    slot, so a reused slot needs no clearing."""
+    normed mixer input (token shift; None for a run without one when ``shift_layers`` says so);
+    ``rec[l]`` ``[n_slots, rec_width_l]`` the state of the layer's recurrence — a channel vector,
+    or the flattened heads x dim x dim matrix state of a wkv mixer (None for a layer without one).
+    A sequence at position 0 never reads its slot, so a reused slot needs no clearing."""
 
     def __init__(self, shapes, width: int, rec_widths, num_blocks: int, block_size: int, device,
-                 dtype=torch.bfloat16, n_slots: int = 16, matrix_layout=None):
+                 dtype=torch.bfloat16, n_slots: int = 16, matrix_layout=None, shift_layers=None):
+        shapes = [sh if sh is not None else (0, 0, 0) for sh in shapes]
         self.n_layers = len(shapes)
         # per run: the layout of the framework's matrix-core attention kernels (keys chunk-major
         # per block, values transposed [.., vdim, block_size]) instead of plain rows
         self.matrix = list(matrix_layout) if matrix_layout is not None else [False] * len(shapes)
         self.shapes = [tuple(int(x) for x in sh) for sh in shapes]
-        self.n_kv_heads = max(sh[0] for sh in self.shapes)
-        self.head_dim = max(max(sh[1], sh[2]) for sh in self.shapes)
+        self.n_kv_heads = max(1, max(sh[0] for sh in self.shapes))
+        self.head_dim = max(1, max(max(sh[1], sh[2]) for sh in self.shapes))
         self.block_size, self.num_blocks = block_size, num_blocks
         self.device, self.dtype = device, dtype
         # zero-init: tail rows of a partial block are masked, never skipped, so they must be finite
-        self.k = [torch.zeros(num_blocks, g, block_size, dk, dtype=dtype, device=device) for g, dk, _ in self.shapes]
-        self.v = [torch.zeros((num_blocks, g, dv, block_size) if mx else (num_blocks, g, block_size, dv), dtype=dtype,
-                              device=device) for (g, _, dv), mx in zip(self.shapes, self.matrix)]
+        self.k = [torch.zeros(num_blocks, g, block_size, dk, dtype=dtype, device=device) if g else None
+                  for g, dk, _ in self.shapes]
+        self.v = [(torch.zeros((num_blocks, g, dv, block_size) if mx else (num_blocks, g, block_size, dv), dtype=dtype,
+                               device=device) if g else None) for (g, _, dv), mx in zip(self.shapes, self.matrix)]
         self.alloc = BlockAllocator(num_blocks)
         self.seqs = {}
         self.state = StateSlots(n_slots)
-        self.shift = [torch.zeros(n_slots, width, dtype=torch.float32, device=device) for _ in self.shapes]
+        shift_layers = list(shift_layers) if shift_layers is not None else [True] * len(self.shapes)
+        self.shift = [torch.zeros(n_slots, width, dtype=torch.float32, device=device) if on else None
+                      for on in shift_layers]
         self.rec = [torch.zeros(n_slots, w, dtype=torch.float32, device=device) if w else None for w in rec_widths]
 
     @staticmethod
@@ -340,7 +348,8 @@ class GroupedKVCache(StatefulPagedCache):
         si = torch.tensor(src, dtype=torch.int64, device=self.device)
         di = torch.tensor(dst, dtype=torch.int64, device=self.device)
         for t in self.k + self.v:
-            t.index_copy_(0, di, t.index_select(0, si))
+            if t is not None:
+                t.index_copy_(0, di, t.index_select(0, si))
 
     def state_tensors(self) -> List[torch.Tensor]:
-        return self.shift + [r for r in self.rec if r is not None]
+        return [t for t in self.shift + self.rec if t is not None]

@@ -45,7 +45,14 @@ class GroupedAttentionSpec:
     denominator as exp(0) * sink: a key of score 0 without a value (0 = ordinary softmax).
     ``head_temp``: every head multiplies its scores by a learned number (tensor ``temp``).
     ``value_from_key``: there is no value projection, the values are the projected keys as they
-    are before the norm."""
+    are before the norm.
+    ``window`` > 0: position i sees only j with 0 <= i - j < window. ``slope_base`` > 0: head a
+    takes slope_a * (i - j) off its scores, slope_a = 2^(-slope_base * (a + 1) / heads).
+    ``qk_weight``: the query / key norms multiply by a learned weight per channel (tensors
+    ``q.norm`` / ``k.norm``, shared by the heads). ``q_temp`` = (coef, every): the queries of
+    position p are multiplied by 1 + coef * ln(floor((p + 1) / every) + 1). ``value_norm``: every
+    value head is divided by its root mean square before it is cached. ``out_gate``: the
+    concatenated heads are multiplied by sigmoid(W_g h) ahead of the output projection."""
     heads: int
     kv_heads: int
     dim: int
@@ -55,6 +62,12 @@ class GroupedAttentionSpec:
     sink: float = 0.0
     head_temp: bool = False
     value_from_key: bool = False
+    window: int = 0
+    slope_base: float = 0.0
+    qk_weight: bool = False
+    q_temp: Optional[Tuple[float, int]] = None
+    value_norm: bool = False
+    out_gate: bool = False
 
     @property
     def group(self) -> int:
@@ -82,16 +95,48 @@ class ParallelSpec:
 
 
 @dataclass(frozen=True)
+class WKVSpec:
+    """Linear-attention time mixing with a per-token, per-channel decay (RWKV style): ``heads``
+    heads whose keys and values are ``dim`` wide, a ``dim`` x ``dim`` fp32 state per head, and a
+    low-rank path of width ``decay_rank`` from the shifted input to the decay's logarithm."""
+    heads: int
+    dim: int
+    decay_rank: int
+
+    @property
+    def width(self) -> int:
+        return self.heads * self.dim
+
+    @property
+    def state_size(self) -> int:
+        """fp32 numbers of the recurrent state per sequence."""
+        return self.heads * self.dim * self.dim
+
+
+@dataclass(frozen=True)
+class MoESpec:
+    """Mixture of gated feed-forward experts: ``experts`` experts of width ``ff``, each token runs
+    the ``top`` with the largest router logits, weighted by the softmax over those logits alone."""
+    experts: int
+    top: int
+    ff: int
+
+
+@dataclass(frozen=True)
 class LayerSpec:
     """One decoder layer of a per-layer-configured model: its mixer, its feed-forward (``ff`` 0 =
     none) and ``source``, the layer whose tensors it uses (itself unless its weights are shared).
-    ``ff_limit``: the clamp of a limited gated feed-forward."""
+    ``ff_limit``: the clamp of a limited gated feed-forward. ``moe``: the experts of a
+    feed-forward of kind "moe" (``ff`` is then one expert's width). ``opens_pass``: this run is the
+    first of pass number ``opens_pass`` of a looped span (None: it opens none)."""
     mixer_type: str
     mixer: object
     ff: int
     ff_kind: str
     source: int
     ff_limit: float = 0.0
+    moe: Optional[MoESpec] = None
+    opens_pass: Optional[int] = None
 
 
 @dataclass(frozen=True)
@@ -120,6 +165,8 @@ class ModelConfig:
     logit_scale: float = 1.0
     logit_softcap: float = 0.0
     embed_scale: float = 1.0      # the embedding row is multiplied by it ("goganex")
+    norm_groups: int = 1          # RMS norms of the residual stream work on this many equal parts ("retuvik")
+    loop_passes: int = 0          # passes of the looped span that add the embedding / a step vector ("retuvik")
 
     @property
     def q_size(self) -> int:
@@ -135,13 +182,13 @@ class ModelConfig:
 
     def n_params(self) -> int:
         h, f, v, L = self.hidden, self.ffn, self.vocab, self.n_layers
-        if self.arch == "goganex":
-            from .weights import goganex_layout
+        if self.arch in ("goganex", "retuvik"):
+            from .weights import layout_for
             n = 0
-            for shape, _, _ in goganex_layout(self).values():
+            for shape, _, _ in layout_for(self).values():
                 k = 1
                 for d in shape:
-                    k *= d
+                    k *= d if d >= 0 else 32
                 n += k
             return n
         if self.layers is not None:
@@ -167,7 +214,7 @@ class ModelConfig:
 
     def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
         if self.layers is not None:
-            return sum(attention_of(ls).cache_row for ls in self.layers) * dtype_bytes
+            return sum(attention_of(ls).cache_row for ls in self.layers if attention_of(ls) is not None) * dtype_bytes
         return 2 * self.n_layers * self.n_kv_heads * self.head_dim * dtype_bytes
 
 
@@ -241,7 +288,10 @@ def parse_mupulorn(d: dict, name: str = "mupulorn") -> ModelConfig:
 
 
 def attention_of(ls: LayerSpec):
-    """The attention part of a layer's mixer (the left half of a parallel mixer)."""
+    """The attention part of a layer's mixer (the left half of a parallel mixer; None for a
+    mixer without attention)."""
+    if isinstance(ls.mixer, WKVSpec):
+        return None
     return ls.mixer.left if isinstance(ls.mixer, ParallelSpec) else ls.mixer
 
 
@@ -321,6 +371,94 @@ def goganex_config(name: str, n_layers: int, width: int, heads: int, kv_heads: i
     return parse_goganex(d, name)
 
 
+
+def parse_retuvik(d: dict, name: str = "retuvik") -> ModelConfig:
+    """``config.json`` of a Retuvik checkpoint -> :class:`ModelConfig`. ``layers`` of the result are
+    the layer RUNS in execution order: checkpoint layers ``loop.start .. loop.stop - 1`` run
+    ``loop.times`` times in a row with the same tensors, every run with a cache and state of its
+    own; the first run of pass t is marked ``opens_pass = t`` (the model adds the embedding output
+    again from the second pass on, and row t of ``loop.step`` in every pass). A key the file does
+    not have switches its mechanism off (no window, no query factor, no loop). The width of a wkv
+    mixer's low-rank decay path is a tensor shape, not a config key: ``mixer.decay_rank`` is read
+    only by random initialisation."""
+    raw = d["layers"]
+    runs = [(i, None) for i in range(len(raw))]
+    lp = d.get("loop")
+    passes = 0
+    if lp is not None:
+        a, b, passes = int(lp["start"]), int(lp["stop"]), int(lp["times"])
+        if not (0 <= a <= b <= len(raw)) or passes < 1:
+            raise ValueError(f"{name}: loop {lp} does not fit {len(raw)} layers")
+        if a == b:
+            passes = 0
+        body = [[(i, t if i == a else None) for i in range(a, b)] for t in range(passes)]
+        runs = runs[:a] + sum(body, []) + runs[b:]
+    specs = []
+    for i, opens in runs:
+        e, where = raw[i], f"{name}: layer {i}"
+        mx = e["mixer"]
+        if e["type"] == "wkv":
+            mixer = WKVSpec(int(mx["heads"]), int(mx["dim"]), int(mx.get("decay_rank", 0)))
+        elif e["type"] == "attention":
+            qt, mask = mx.get("q_temp"), mx.get("mask")
+            mixer = _grouped_attention(mx, where, window=int(mask["size"]) if mask is not None else 0, slope_base=8.0,
+                                       qk_weight=True, value_norm=True, out_gate=True,
+                                       q_temp=(float(qt["coef"]), int(qt["every"])) if qt is not None else None)
+            if mixer.window < 0 or (mixer.q_temp is not None and mixer.q_temp[1] < 1):
+                raise ValueError(f"{where}: mask.size / q_temp.every out of range")
+        else:
+            raise ValueError(f"{where}: unknown mixer type '{e['type']}'")
+        mlp = e.get("mlp")
+        if mlp is None:
+            specs.append(LayerSpec(e["type"], mixer, 0, "dense", i, opens_pass=opens))
+        elif mlp.get("kind", "dense") == "dense":
+            specs.append(LayerSpec(e["type"], mixer, int(mlp["ff"]), "dense", i, opens_pass=opens))
+        elif mlp["kind"] == "moe":
+            moe = MoESpec(int(mlp["router"]["experts"]), int(mlp["router"]["top"]), int(mlp["expert"]["ff"]))
+            if not 1 <= moe.top <= moe.experts:
+                raise ValueError(f"{where}: top {moe.top} of {moe.experts} experts")
+            specs.append(LayerSpec(e["type"], mixer, moe.ff, "moe", i, moe=moe, opens_pass=opens))
+        else:
+            raise ValueError(f"{where}: unknown feed-forward kind '{mlp['kind']}'")
+    width, groups = int(d["width"]), int(d["norm"].get("groups", 1))
+    if groups < 1 or width % groups:
+        raise ValueError(f"{name}: width {width} does not split into {groups} norm groups")
+    atts = [s.mixer for s in specs if isinstance(s.mixer, GroupedAttentionSpec)]
+    top = max(atts, key=lambda m: m.heads) if atts else None
+    any_mixer = specs[0].mixer
+    return ModelConfig(name, "retuvik", len(specs), width, top.heads if top else any_mixer.heads,
+                       top.kv_heads if top else any_mixer.heads, top.dim if top else any_mixer.dim,
+                       max([s.ff for s in specs] + [0]), int(d["vocab"]), int(d.get("max_pos", 1 << 17)), 0.0,
+                       float(d["norm"]["eps"]), layers=tuple(specs),
+                       embed_scale=float(d.get("embedding", {}).get("scale", 1.0)), norm_groups=groups,
+                       loop_passes=passes)
+
+
+def retuvik_config(name: str, n_layers: int, width: int, heads: int, kv_heads: int, dim: int, ff: int, vocab: int,
+                   attention_every: int = 3, wkv_dim: int = 64, decay_rank: int = 64, window: int = 1024,
+                   moe_every: int = 0, experts: int = 8, top: int = 2, expert_ff: int = 0,
+                   loop: Optional[Tuple[int, int, int]] = None, groups: int = 2, max_pos: int = 1 << 17) -> ModelConfig:
+    """A Retuvik stack from a few sizes (benchmarks and presets): wkv layers with every
+    ``attention_every``-th layer a windowed attention layer (0: none); every ``moe_every``-th
+    feed-forward a mixture of experts (0: all dense)."""
+    wkv = {"type": "wkv", "mixer": {"heads": width // wkv_dim, "dim": wkv_dim, "decay_rank": decay_rank}}
+    att = {"type": "attention",
+           "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                     "mask": {"size": window}, "q_temp": {"coef": 0.1, "every": 1024}}}
+    dense = {"kind": "dense", "ff": ff} if ff else None
+    moe = {"kind": "moe", "expert": {"ff": expert_ff or ff // top}, "router": {"experts": experts, "top": top}}
+    layers = []
+    for i in range(n_layers):
+        e = dict(att if attention_every and (i + 1) % attention_every == 0 else wkv)
+        e["mlp"] = moe if moe_every and (i + 1) % moe_every == 0 else dense
+        layers.append(e)
+    d = {"architecture": "Retuvik", "embedding": {"scale": 1.0}, "layers": layers, "norm": {"eps": 1e-5, "groups": groups},
+         "vocab": vocab, "width": width, "max_pos": max_pos}
+    if loop is not None:
+        d["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
+    return parse_retuvik(d, name)
+
+
 def mupulorn_config(name: str, n_layers: int, width: int, heads: int, dim: int, rot_dim: int, vdim: int,
                     kv_rank: int, q_rank: int, ff: int, vocab: int, taps: int = 4, shared_every: int = 0,
                     rot_base: float = 10000.0, max_pos: int = 1 << 17) -> ModelConfig:
@@ -343,7 +481,8 @@ def mupulorn_config(name: str, n_layers: int, width: int, heads: int, dim: int, 
 
 
 # config.json "architecture" -> parser (checkpoint directories name their own model class)
-ARCHITECTURES: Dict[str, Callable[[dict, str], ModelConfig]] = {"Mupulorn": parse_mupulorn, "Goganex": parse_goganex}
+ARCHITECTURES: Dict[str, Callable[[dict, str], ModelConfig]] = {"Mupulorn": parse_mupulorn, "Goganex": parse_goganex,
+                                                                "Retuvik": parse_retuvik}
 
 PRESETS.update({
     # Mupulorn (latent attention + input convolutions + PolyNorm feed-forward), random-init sizes:
@@ -367,6 +506,19 @@ PRESETS.update({
     "goganex-1b": goganex_config("goganex-1b", 16, 2048, 32, 8, 64, 8192, 128256),
     "goganex-3b": goganex_config("goganex-3b", 28, 3072, 24, 8, 128, 8192, 128256),
     "goganex-8b": goganex_config("goganex-8b", 32, 4096, 32, 8, 128, 14336, 128256),
+})
+
+PRESETS.update({
+    # Retuvik (wkv time mixing with a per-token decay, windowed attention with a distance penalty,
+    # xIELU and mixture-of-experts feed-forwards, grouped RMS norms), random-init sizes: a test-sized
+    # stack with a looped middle, and stacks whose layers have the shapes of 1B / 3B / 8B-class Llama
+    # models (every third layer attention, every fourth feed-forward a mixture of 8 experts, 2 per token)
+    "tiny-retuvik": retuvik_config("tiny-retuvik", 4, 128, 4, 2, 32, 256, 32000, attention_every=2, wkv_dim=32,
+                                   decay_rank=16, window=24, moe_every=2, experts=6, top=2, expert_ff=64,
+                                   loop=(1, 3, 2)),
+    "retuvik-1b": retuvik_config("retuvik-1b", 16, 2048, 32, 8, 64, 8192, 128256, moe_every=4),
+    "retuvik-3b": retuvik_config("retuvik-3b", 28, 3072, 24, 8, 128, 8192, 128256, moe_every=4),
+    "retuvik-8b": retuvik_config("retuvik-8b", 32, 4096, 32, 8, 128, 14336, 128256, moe_every=4),
 })
 
 

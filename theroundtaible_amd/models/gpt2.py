@@ -92,5 +92,8 @@ def build_model(cfg: ModelConfig, weights, device, dtype=torch.bfloat16, tp: Opt
     if cfg.arch == "goganex":
         from .goganex import GoganexModel
         return GoganexModel(cfg, weights, device, dtype, tp)
+    if cfg.arch == "retuvik":
+        from .retuvik import RetuvikModel
+        return RetuvikModel(cfg, weights, device, dtype, tp)
     from .llama import LlamaModel
     return LlamaModel(cfg, weights, device, dtype, tp)

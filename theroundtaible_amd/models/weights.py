@@ -152,11 +152,72 @@ def goganex_layout(cfg: ModelConfig) -> Dict[str, Tuple[Tuple[int, ...], str, Op
     return lay
 
 
+def retuvik_layout(cfg: ModelConfig) -> Dict[str, Tuple[Tuple[int, ...], str, Optional[str]]]:
+    """Checkpoint names and shapes of a Retuvik model (linear weights [out, in]). A looped layer has
+    one set of tensors, named by its place in the checkpoint's layer list. The rank of a wkv
+    mixer's decay path is whatever ``mix.w1`` / ``mix.w2`` have (-1 in the shape) unless the spec
+    names one. Not tensor-parallel: every kind is None."""
+    from .config import WKVSpec
+    W = cfg.hidden
+    lay: Dict[str, Tuple[Tuple[int, ...], str, Optional[str]]] = {
+        "embed": ((cfg.vocab, W), "normal", None),
+        "final.norm": ((W,), "ones", None),
+        "head": ((cfg.vocab, W), "normal", None),
+    }
+    if cfg.loop_passes:
+        lay["loop.step"] = ((cfg.loop_passes, W), "normal", None)
+    for ls in cfg.layers:
+        p = f"l{ls.source}."
+        if p + "norm1" in lay:
+            continue
+        lay[p + "norm1"] = ((W,), "ones", None)
+        m = ls.mixer
+        if isinstance(m, WKVSpec):
+            rank = m.decay_rank or -1
+            for n in "rkvgw":
+                lay[p + "mix.mu." + n] = ((W,), "half", None)
+            for n in "rkvg":
+                lay[p + "mix." + n] = ((m.width, W), "normal", None)
+            lay[p + "mix.w1"] = ((rank, W), "normal", None)
+            lay[p + "mix.w2"] = ((m.width, rank), "normal", None)
+            lay[p + "mix.w0"] = ((m.width,), "zeros", None)
+            lay[p + "mix.u"] = ((m.heads, m.dim), "small", None)
+            lay[p + "mix.norm"] = ((m.width,), "ones", None)
+            lay[p + "mix.o"] = ((W, m.width), "normal", None)
+        else:
+            lay[p + "mix.q"] = ((m.heads * m.dim, W), "normal", None)
+            lay[p + "mix.k"] = ((m.kv_heads * m.dim, W), "normal", None)
+            lay[p + "mix.v"] = ((m.kv_heads * m.vdim, W), "normal", None)
+            lay[p + "mix.q.norm"] = ((m.dim,), "ones", None)
+            lay[p + "mix.k.norm"] = ((m.dim,), "ones", None)
+            lay[p + "mix.g"] = ((m.heads * m.vdim, W), "normal", None)
+            lay[p + "mix.o"] = ((W, m.heads * m.vdim), "normal", None)
+        if not ls.ff:
+            continue
+        lay[p + "norm2"] = ((W,), "ones", None)
+        if ls.ff_kind == "moe":
+            for e in range(ls.moe.experts):
+                lay[p + f"mlp.e{e}.gate"] = ((ls.ff, W), "normal", None)
+                lay[p + f"mlp.e{e}.up"] = ((ls.ff, W), "normal", None)
+                lay[p + f"mlp.e{e}.down"] = ((W, ls.ff), "normal", None)
+            lay[p + "mlp.router"] = ((ls.moe.experts, W), "normal", None)
+            lay[p + "mlp.router.b"] = ((ls.moe.experts,), "zeros", None)
+        else:
+            lay[p + "mlp.up"] = ((ls.ff, W), "normal", None)
+            lay[p + "mlp.up.b"] = ((ls.ff,), "zeros", None)
+            lay[p + "mlp.down"] = ((W, ls.ff), "normal", None)
+            lay[p + "mlp.down.b"] = ((W,), "zeros", None)
+            lay[p + "mlp.act"] = ((2,), "zeros", None)
+    return lay
+
+
 def layout_for(cfg: ModelConfig):
     if cfg.arch == "mupulorn":
         return mupulorn_layout(cfg)
     if cfg.arch == "goganex":
         return goganex_layout(cfg)
+    if cfg.arch == "retuvik":
+        return retuvik_layout(cfg)
     return gpt2_layout(cfg) if cfg.arch == "gpt2" else llama_layout(cfg)
 
 
@@ -232,6 +293,7 @@ def materialize(cfg: ModelConfig, spec: str, device, dtype=torch.bfloat16, tp: O
 
 
 def _init(shape, init, std, g, device, dtype):
+    shape = tuple(32 if n < 0 else n for n in shape)     # a size the checkpoint alone would fix
     if init == "ones":
         return torch.ones(shape, device=device, dtype=dtype)
     if init == "zeros":
@@ -310,7 +372,7 @@ def load_safetensors(cfg: ModelConfig, path: str, device, dtype, tp: TPInfo) -> 
         tensors.update(load_file(f, device="cpu"))
     lay = layout_for(cfg)
     out = {}
-    if cfg.arch in ("mupulorn", "goganex"):
+    if cfg.arch in ("mupulorn", "goganex", "retuvik"):
         # the checkpoint's own names; integer tables keep their type, everything else takes `dtype`
         if tp.size > 1:
             raise ValueError(f"{cfg.arch} checkpoints are not tensor-parallel")
@@ -318,7 +380,7 @@ def load_safetensors(cfg: ModelConfig, path: str, device, dtype, tp: TPInfo) -> 
             if name not in tensors:
                 raise KeyError(f"{path}: tensor '{name}' is missing")
             w = tensors[name]
-            if tuple(w.shape) != tuple(shape):
+            if len(w.shape) != len(shape) or any(b >= 0 and a != b for a, b in zip(w.shape, shape)):
                 raise ValueError(f"{path}: tensor '{name}' has shape {tuple(w.shape)}, config.json gives {tuple(shape)}")
             out[name] = (w if not w.is_floating_point() else w.to(dtype)).to(device).contiguous()
         return out

@@ -1,8 +1,11 @@
 """Ops of decoders that mix grouped attention with recurrent layers: token shift fused with the
-RMS norm ahead of a mixer, query / key preparation (rotary pairs, per-head unit RMS) with the paged
-cache write, grouped-query attention with an optional softmax sink and per-head temperature, the
-minGRU scan, the two-branch normed residual add, residual add + RMS norm, and the clamped gated
-feed-forward activation.
+RMS norm ahead of a mixer (one or several mixes of the same row; the norm over the whole row or over
+equal parts of it), query / key preparation (rotary pairs, per-head unit RMS, optional weights, a
+query factor that grows with the position, unit-RMS values) with the paged cache write,
+grouped-query attention with an optional softmax sink, per-head temperature, sliding window,
+distance penalty and output gate, the minGRU scan, the wkv scan (linear attention with a per-token
+decay), the two-branch normed residual add, residual add + RMS norm, the clamped gated, xIELU and
+silu-gated feed-forward activations, and a routed mixture of experts.
 
 GPU tensors go to the HIP kernels of ``theroundtaible_amd._C_hybrid`` (``csrc/hybrid/``, built
 in-tree by ``csrc/build.py``; :func:`ensure_built` compiles it on first use in a fresh checkout);
@@ -62,30 +65,32 @@ def _gpu(t: torch.Tensor) -> bool:
 # ---- token shift + norm ---------------------------------------------------------------------------
 
 def shift_norm(x, y, w, eps, mu, state, row_seq, positions, start_pos, slots, out_dtype,
-               shift_state: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+               shift_state: bool = False, groups: int = 1) -> Tuple[torch.Tensor, torch.Tensor]:
     """``x`` [T, W] fp32 residual, ``y`` an optional pending branch output still to be added.
     With ``xs = x + y`` and ``h_r = xs_r / rms(xs_r) * w``: returns ``(h_r + (p_r - h_r) * mu, xs)``
     where ``p_r`` is the previous token's ``h``: row r - 1 inside a span, ``state[slot]`` for the
     first row of a span that continues a sequence, zeros at position 0. ``xs`` is a new tensor
     when ``y`` is given (other rows of the launch still read the old ``x``), else ``x`` itself.
     ``shift_state`` (only with ONE row per sequence, a decode step): the same launch also stores
-    ``h_r`` as the sequence's new state, so no :func:`shift_state_update` follows."""
+    ``h_r`` as the sequence's new state, so no :func:`shift_state_update` follows.
+    ``mu`` [n, W] gives n mixes of the same row at once, returned as [n, T, W]. ``groups`` > 1:
+    the norm divides each of that many equal consecutive parts of a row by its own RMS."""
     if _gpu(x):
-        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        out = torch.empty((mu.shape[0],) + tuple(x.shape) if mu.dim() == 2 else x.shape, dtype=out_dtype, device=x.device)
         xs = torch.empty_like(x) if y is not None else x
         native().shift_norm(out, xs, x, y, w, float(eps), mu, state, row_seq, positions, start_pos, slots,
-                            bool(shift_state))
+                            bool(shift_state), int(groups))
         return out, xs
-    return ref_shift_norm(x, y, w, eps, mu, state, row_seq, positions, start_pos, slots, out_dtype, shift_state)
+    return ref_shift_norm(x, y, w, eps, mu, state, row_seq, positions, start_pos, slots, out_dtype, shift_state, groups)
 
 
-def shift_state_update(x, w, eps, state, cu_q, slots) -> None:
+def shift_state_update(x, w, eps, state, cu_q, slots, groups: int = 1) -> None:
     """Store the normed last row of every span as its sequence's state. Runs AFTER
     :func:`shift_norm` of the same layer (it overwrites what that one reads)."""
     if _gpu(x):
-        native().shift_state_update(x, w, float(eps), state, cu_q, slots)
+        native().shift_state_update(x, w, float(eps), state, cu_q, slots, int(groups))
         return
-    ref_shift_state_update(x, w, eps, state, cu_q, slots)
+    ref_shift_state_update(x, w, eps, state, cu_q, slots, groups)
 
 
 # ---- queries, keys, values ------------------------------------------------------------------------
@@ -100,7 +105,8 @@ def rotary_table(rot, device) -> Optional[torch.Tensor]:
 
 
 def qk_prep(proj, spec, q_off: int, k_off: int, v_off: int, inv_freq, eps, positions, k_cache, v_cache,
-            slot_mapping, out_dtype, matrix_layout: bool = False, q_scale=None) -> torch.Tensor:
+            slot_mapping, out_dtype, matrix_layout: bool = False, q_scale=None, q_weight=None,
+            k_weight=None) -> torch.Tensor:
     """``proj`` [T, N]: columns ``q_off ..`` hold the projected queries (heads x dim), ``k_off ..``
     the keys (kv_heads x dim), ``v_off ..`` the values (kv_heads x vdim; ignored when the values
     are the keys). Rotates the leading ``2 * len(inv_freq)`` entries of every query / key head
@@ -108,19 +114,24 @@ def qk_prep(proj, spec, q_off: int, k_off: int, v_off: int, inv_freq, eps, posit
     mean square, writes keys and values to the paged cache at ``slot_mapping`` and returns the
     queries [T, heads, dim]. ``matrix_layout`` (GPU): the cache of the framework's matrix-core
     attention kernels — keys chunk-major per block, values transposed ``[nb, G, vdim, BS]``;
-    ``q_scale`` [heads] fp32 multiplies each query head (a per-head temperature moved into q)."""
+    ``q_scale`` [heads] fp32 multiplies each query head (a per-head temperature moved into q).
+    ``q_weight`` / ``k_weight`` [dim] fp32 multiply the normed queries / keys channel by channel.
+    ``spec.q_temp`` = (coef, every): queries of position p times 1 + coef ln(floor((p + 1) / every) + 1);
+    ``spec.value_norm``: every value head is divided by its root mean square before it is cached."""
     if _gpu(proj):
         T = proj.shape[0]
         q = torch.empty(T, spec.heads, spec.dim, dtype=out_dtype, device=proj.device)
+        qt = spec.q_temp or (0.0, 0)
         native().qk_prep(q, proj, int(q_off), int(k_off), int(v_off), bool(spec.value_from_key), inv_freq, float(eps),
-                         positions, k_cache, v_cache, slot_mapping, 1 if matrix_layout else 0, q_scale)
+                         positions, k_cache, v_cache, slot_mapping, 1 if matrix_layout else 0, q_scale, q_weight, k_weight,
+                         bool(spec.value_norm), float(qt[0]), int(qt[1]))
         return q
     if matrix_layout:
         raise ValueError("qk_prep: the matrix-core cache layout exists on the GPU only")
     if q_scale is not None:
         raise ValueError("qk_prep: q_scale is a GPU-path option (the CPU statement keeps the temperature in the scores)")
     return ref_qk_prep(proj, spec, q_off, k_off, v_off, inv_freq, eps, positions, k_cache, v_cache, slot_mapping,
-                       out_dtype)
+                       out_dtype, q_weight, k_weight)
 
 
 def rows_per_tile(group: int) -> int:
@@ -151,13 +162,15 @@ class SplitWorkspace:
 
 def gqa_attention(q, k_cache, v_cache, block_tables, cu_q, start_pos, scale: float, temp=None, sink: float = 0.0,
                   tiles=None, num_splits: int = 1, workspace: Optional[SplitWorkspace] = None,
-                  out_dtype=None) -> torch.Tensor:
+                  out_dtype=None, window: int = 0, slopes=None, gate=None, gate_off: int = 0) -> torch.Tensor:
     """Causal attention of the rows ``q`` [T, H, Dk] (span s = rows ``cu_q[s] .. cu_q[s + 1]`` at
     positions ``start_pos[s] ..`` of sequence s) over the paged keys ``k_cache`` [nb, G, BS, Dk]
     and values ``v_cache`` [nb, G, BS, Dv]: score = q . k * scale (* ``temp[h]``), weights
     exp(s_j) / (``sink`` + sum exp(s_j)). Returns [T, H * Dv]. ``tiles``: :func:`tile_map` on the
     device; ``num_splits`` > 1 (one row per span: a decode step) cuts every row's keys into that
-    many ranges merged by a second launch."""
+    many ranges merged by a second launch. ``window`` > 0: row i sees only keys j with
+    i - j < window. ``slopes`` [H] fp32: head h takes slopes[h] * (i - j) off its scores. ``gate``
+    [T, N]: the result is multiplied by sigmoid of its columns ``gate_off .. gate_off + H * Dv``."""
     out_dtype = out_dtype or q.dtype
     if _gpu(q):
         T, H, _ = q.shape
@@ -171,9 +184,10 @@ def gqa_attention(q, k_cache, v_cache, block_tables, cu_q, start_pos, scale: flo
         native().gqa_attention(out, q, k_cache, v_cache, block_tables, cu_q, start_pos, tiles, temp, float(scale),
                                float(sink), rows, int(num_splits),
                                workspace.part_o if num_splits > 1 else None,
-                               workspace.part_ml if num_splits > 1 else None)
+                               workspace.part_ml if num_splits > 1 else None, int(window), slopes, gate, int(gate_off))
         return out
-    return ref_gqa_attention(q, k_cache, v_cache, block_tables, cu_q, start_pos, scale, temp, sink, out_dtype)
+    return ref_gqa_attention(q, k_cache, v_cache, block_tables, cu_q, start_pos, scale, temp, sink, out_dtype,
+                             window, slopes, gate, gate_off)
 
 
 # ---- minGRU ---------------------------------------------------------------------------------------
@@ -227,13 +241,14 @@ def dual_norm_add_(x, a, wa, b, wb, eps) -> torch.Tensor:
     return ref_dual_norm_add_(x, a, wa, b, wb, eps)
 
 
-def add_norm(x, y, w, eps, out_dtype) -> torch.Tensor:
-    """x += y (in place, fp32; ``y`` may be None), returns x / rms(x) * w."""
+def add_norm(x, y, w, eps, out_dtype, groups: int = 1) -> torch.Tensor:
+    """x += y (in place, fp32; ``y`` may be None), returns x / rms(x) * w; with ``groups`` > 1 each
+    of that many equal consecutive parts of a row is divided by its own RMS."""
     if _gpu(x):
         out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
-        native().add_norm(out, x, y, w, float(eps))
+        native().add_norm(out, x, y, w, float(eps), int(groups))
         return out
-    return ref_add_norm(x, y, w, eps, out_dtype)
+    return ref_add_norm(x, y, w, eps, out_dtype, groups)
 
 
 def limited_glu(gu, limit: float, out_dtype) -> torch.Tensor:
@@ -246,30 +261,140 @@ def limited_glu(gu, limit: float, out_dtype) -> torch.Tensor:
     return ref_limited_glu(gu, limit, out_dtype)
 
 
+# ---- wkv ------------------------------------------------------------------------------------------
+
+WKV_CHUNK = 64           # rows per chunk of the chunked wkv scan (csrc/hybrid/hybrid_wkv.hip kWkvChunk)
+
+
+def wkv_chunks(cu_q: torch.Tensor, device=None, min_rows: int = 2 * WKV_CHUNK):
+    """Work lists of the chunked wkv scan, as :func:`scan_chunks`: None when no span has more than
+    ``min_rows`` rows (the one-launch scan is used then)."""
+    cq = cu_q.tolist()
+    if max((b - a for a, b in zip(cq, cq[1:])), default=0) <= min_rows:
+        return None
+    chunks, first = [], [0]
+    for s in range(len(cq) - 1):
+        chunks += [(s, r) for r in range(cq[s], cq[s + 1], WKV_CHUNK)]
+        first.append(len(chunks))
+    return (torch.tensor(chunks, dtype=torch.int32).reshape(-1, 2).to(device, non_blocking=True),
+            torch.tensor(first, dtype=torch.int32).to(device, non_blocking=True))
+
+
+def wkv_scan(rkvg, lw, w0, u, norm_w, eps, state, cu_q, start_pos, slots, out_dtype, chunks=None) -> torch.Tensor:
+    """``rkvg`` [4, T, H * D]: the projected r, k, v and output gate; ``lw`` [T, H * D] the decay's
+    low-rank path; ``w0`` [H * D], ``u`` [H, D], ``norm_w`` [H * D] fp32. Per sequence and head,
+    with the D x D state S from ``state[slot]`` [H * D * D] (zeros at position 0), in fp32:
+        decay = exp(-exp(lw + w0));  o_t[j] = sum_i r_t[i] (S[i, j] + u[i] k_t[i] v_t[j]);
+        S[i, j] <- decay_t[i] S[i, j] + k_t[i] v_t[j]
+    and returns o_t / rms(o_t per head) * norm_w * silu(gate_t) [T, H * D]; every span's last S is
+    left in ``state``. ``chunks`` (GPU): :func:`wkv_chunks` of this batch — spans are then scanned
+    in chunks in parallel (chunk end states and decay products, a carry pass, the outputs from each
+    chunk's true start state); the results differ from the one-launch scan by rounding only."""
+    if _gpu(rkvg):
+        out = torch.empty(rkvg.shape[1], rkvg.shape[2], dtype=out_dtype, device=rkvg.device)
+        if chunks is not None:
+            H, D = u.shape
+            ws = torch.empty(chunks[0].shape[0] * H * (2 * D * D + D), dtype=torch.float32, device=rkvg.device)
+            native().wkv_scan(out, rkvg, lw, w0, u, norm_w, float(eps), state, cu_q, start_pos, slots, chunks[0], chunks[1], ws)
+        else:
+            native().wkv_scan(out, rkvg, lw, w0, u, norm_w, float(eps), state, cu_q, start_pos, slots)
+        return out
+    return ref_wkv_scan(rkvg, lw, w0, u, norm_w, eps, state, cu_q, start_pos, slots, out_dtype)
+
+
+# ---- feed-forward -----------------------------------------------------------------------------------
+
+def xielu(a, bias, alpha_pos: float, alpha_neg: float, out_dtype) -> torch.Tensor:
+    """z = a + bias; alpha_pos z^2 + z / 2 for z > 0, alpha_neg (e^z - 1 - z) + z / 2 otherwise."""
+    if _gpu(a):
+        out = torch.empty(a.shape, dtype=out_dtype, device=a.device)
+        native().xielu(out, a, bias, float(alpha_pos), float(alpha_neg))
+        return out
+    return ref_xielu(a, bias, alpha_pos, alpha_neg, out_dtype)
+
+
+def silu_glu(gu, out_dtype) -> torch.Tensor:
+    """``gu`` [T, 2F] = (gate | up): silu(gate) * up."""
+    if _gpu(gu):
+        out = torch.empty(gu.shape[0], gu.shape[1] // 2, dtype=out_dtype, device=gu.device)
+        native().silu_glu(out, gu)
+        return out
+    return ref_silu_glu(gu, out_dtype)
+
+
+def topk_softmax(logits, top: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per row of fp32 ``logits`` [T, E]: the indices [T, top] int32 of the ``top`` largest (largest
+    first) and the softmax over those alone [T, top] fp32."""
+    if _gpu(logits) and logits.shape[1] <= 512 and top <= 64:
+        idx = torch.empty(logits.shape[0], top, dtype=torch.int32, device=logits.device)
+        wt = torch.empty(logits.shape[0], top, dtype=torch.float32, device=logits.device)
+        native().topk_softmax(idx, wt, logits.contiguous())
+        return idx, wt
+    val, idx = torch.topk(logits, top, dim=-1)
+    return idx.to(torch.int32), torch.softmax(val, dim=-1)
+
+
+MOE_ROWS = 16            # steps of up to this many rows run the experts row by row (moe_rows)
+
+
+def moe_experts(h, idx, wt, w_gu, w_down, out_dtype, by_row: Optional[bool] = None) -> torch.Tensor:
+    """Mixture of gated experts: ``h`` [T, W]; row t runs experts ``idx[t]`` [top] and adds their
+    outputs W_down[e] (silu(W_gate[e] h) * (W_up[e] h)) with the weights ``wt[t]``. ``w_gu``
+    [E, 2F, W] = every expert's gate rows, then up rows; ``w_down`` [E, W, F]. Two forms: row by row
+    (GPU steps of a few rows: two launches, no host round trip, so a captured decode step can hold
+    them) and expert by expert (the rows of each expert gathered for library GEMMs, one host read of
+    the expert counts; rows are added to the fp32 sum in expert order whatever else is in the batch)."""
+    T, top = idx.shape
+    if by_row is None:
+        by_row = _gpu(h) and T <= MOE_ROWS
+    if by_row and _gpu(h):
+        out = torch.empty(h.shape, dtype=out_dtype, device=h.device)
+        hid = torch.empty(T * top * w_down.shape[2], dtype=torch.float32, device=h.device)
+        native().moe_rows(out, hid, h.contiguous(), w_gu, w_down, idx, wt)
+        return out
+    E = w_gu.shape[0]
+    flat = idx.reshape(-1).long()
+    order = torch.argsort(flat, stable=True)
+    counts = torch.bincount(flat, minlength=E).tolist()
+    rows, cw = order // top, wt.reshape(-1)[order]
+    out = torch.zeros(h.shape, dtype=torch.float32, device=h.device)
+    at = 0
+    for e, n in enumerate(counts):
+        if n:
+            r = rows[at:at + n]
+            a = silu_glu(torch.nn.functional.linear(h.index_select(0, r), w_gu[e]), h.dtype)
+            out.index_add_(0, r, torch.nn.functional.linear(a, w_down[e]).float() * cw[at:at + n, None])
+            at += n
+    return out.to(out_dtype)
+
+
 # ---- the PyTorch statements (CPU tensors; what the kernels are tested against) ---------------------
 
-def _rms(x, eps):
+def _rms(x, eps, groups: int = 1):
+    if groups > 1:
+        return _rms(x.reshape(*x.shape[:-1], groups, x.shape[-1] // groups), eps).reshape(x.shape)
     return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
 
 
-def ref_shift_norm(x, y, w, eps, mu, state, row_seq, positions, start_pos, slots, out_dtype, shift_state=False):
+def ref_shift_norm(x, y, w, eps, mu, state, row_seq, positions, start_pos, slots, out_dtype, shift_state=False,
+                   groups=1):
     xs = x + y.float() if y is not None else x
-    h = _rms(xs, eps) * w
+    h = _rms(xs, eps, groups) * w
     prev = torch.zeros_like(h)
     prev[1:] = h[:-1]
     rs = row_seq.long()
     first = positions == start_pos.long()[rs]
     prev = torch.where(first[:, None], state[slots.long()[rs]], prev)
     prev = torch.where((positions == 0)[:, None], torch.zeros_like(prev), prev)
-    out = h + (prev - h) * mu
+    out = h + (prev - h) * (mu[:, None, :] if mu.dim() == 2 else mu)
     if shift_state:
         state[slots.long()[rs]] = h
     return out.to(out_dtype), xs
 
 
-def ref_shift_state_update(x, w, eps, state, cu_q, slots):
+def ref_shift_state_update(x, w, eps, state, cu_q, slots, groups=1):
     last = cu_q.long()[1:] - 1
-    state[slots.long()] = _rms(x[last], eps) * w
+    state[slots.long()] = _rms(x[last], eps, groups) * w
 
 
 def _rotate_pairs(t, positions, inv_freq):
@@ -284,7 +409,8 @@ def _rotate_pairs(t, positions, inv_freq):
     return out
 
 
-def ref_qk_prep(proj, spec, q_off, k_off, v_off, inv_freq, eps, positions, k_cache, v_cache, slot_mapping, out_dtype):
+def ref_qk_prep(proj, spec, q_off, k_off, v_off, inv_freq, eps, positions, k_cache, v_cache, slot_mapping, out_dtype,
+                q_weight=None, k_weight=None):
     T = proj.shape[0]
     H, G, Dk, Dv = spec.heads, spec.kv_heads, spec.dim, spec.vdim
     q = proj[:, q_off:q_off + H * Dk].float().reshape(T, H, Dk)
@@ -293,14 +419,26 @@ def ref_qk_prep(proj, spec, q_off, k_off, v_off, inv_freq, eps, positions, k_cac
     if inv_freq is not None:
         q, k = _rotate_pairs(q, positions, inv_freq), _rotate_pairs(k, positions, inv_freq)
     q, k = _rms(q, eps), _rms(k, eps)
+    if q_weight is not None:
+        q = q * q_weight
+    if k_weight is not None:
+        k = k * k_weight
+    if spec.q_temp is not None:
+        coef, every = spec.q_temp
+        steps = torch.div(positions.long() + 1, every, rounding_mode="floor").to(torch.float32)
+        q = q * (1.0 + coef * torch.log(steps + 1.0))[:, None, None]
+    v = v.reshape(T, G, Dv)
+    if spec.value_norm:
+        v = _rms(v.float(), eps)
     BS = k_cache.shape[2]
     blk, off = slot_mapping // BS, slot_mapping % BS
     k_cache[blk, :, off] = k.to(k_cache.dtype)
-    v_cache[blk, :, off] = v.reshape(T, G, Dv).to(v_cache.dtype)
+    v_cache[blk, :, off] = v.to(v_cache.dtype)
     return q.to(out_dtype)
 
 
-def ref_gqa_attention(q, k_cache, v_cache, block_tables, cu_q, start_pos, scale, temp, sink, out_dtype):
+def ref_gqa_attention(q, k_cache, v_cache, block_tables, cu_q, start_pos, scale, temp, sink, out_dtype,
+                      window=0, slopes=None, gate=None, gate_off=0):
     T, H, Dk = q.shape
     G, BS, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
     out = torch.empty(T, H, Dv, dtype=torch.float32, device=q.device)
@@ -319,13 +457,21 @@ def ref_gqa_attention(q, k_cache, v_cache, block_tables, cu_q, start_pos, scale,
         qs = q[r0:r1].float().permute(1, 0, 2)                                       # [H, n, Dk]
         sc = torch.einsum("hnd,hkd->hnk", qs, K.repeat_interleave(H // G, 0)) * hs[:, None, None]
         qpos = torch.arange(sp[s], ctx, device=q.device)
-        mask = torch.arange(ctx, device=q.device)[None, :] <= qpos[:, None]
+        dist = qpos[:, None] - torch.arange(ctx, device=q.device)[None, :]
+        mask = dist >= 0
+        if window > 0:
+            mask = mask & (dist < window)
+        if slopes is not None:
+            sc = sc - slopes.float()[:, None, None] * dist.to(torch.float32)[None]
         sc = sc.masked_fill(~mask[None], float("-inf"))
         m = sc.max(-1, keepdim=True).values
         e = torch.exp(sc - m)
         den = e.sum(-1, keepdim=True) + sink * torch.exp(-m)
         out[r0:r1] = torch.einsum("hnk,hkd->hnd", e / den, V.repeat_interleave(H // G, 0)).permute(1, 0, 2)
-    return out.reshape(T, H * Dv).to(out_dtype)
+    out = out.reshape(T, H * Dv)
+    if gate is not None:
+        out = out * torch.sigmoid(gate[:, gate_off:gate_off + H * Dv].float())
+    return out.to(out_dtype)
 
 
 def ref_mingru_scan(proj, z_off, x_off, g_off, width, bz, bx, state, cu_q, start_pos, slots, out_dtype):
@@ -351,10 +497,41 @@ def ref_dual_norm_add_(x, a, wa, b, wb, eps):
     return x
 
 
-def ref_add_norm(x, y, w, eps, out_dtype):
+def ref_add_norm(x, y, w, eps, out_dtype, groups=1):
     if y is not None:
         x.add_(y.float())
-    return (_rms(x, eps) * w).to(out_dtype)
+    return (_rms(x, eps, groups) * w).to(out_dtype)
+
+
+def ref_wkv_scan(rkvg, lw, w0, u, norm_w, eps, state, cu_q, start_pos, slots, out_dtype):
+    T, HD = rkvg.shape[1], rkvg.shape[2]
+    H, D = u.shape
+    r, k, v, g = (rkvg[i].float().reshape(T, H, D) for i in range(4))
+    dec = torch.exp(-torch.exp(lw.float() + w0)).reshape(T, H, D)
+    o = torch.empty(T, H, D, dtype=torch.float32, device=rkvg.device)
+    cq, sp, sl = cu_q.tolist(), start_pos.tolist(), slots.tolist()
+    for s in range(len(sp)):
+        if cq[s + 1] == cq[s]:
+            continue
+        S = (state[sl[s]].reshape(H, D, D).clone() if sp[s] > 0
+             else torch.zeros(H, D, D, dtype=torch.float32, device=rkvg.device))
+        for t in range(cq[s], cq[s + 1]):
+            kv = k[t][:, :, None] * v[t][:, None, :]
+            o[t] = torch.einsum("hi,hij->hj", r[t], S + u[:, :, None] * kv)
+            S = dec[t][:, :, None] * S + kv
+        state[sl[s]] = S.reshape(-1)
+    return (_rms(o, eps).reshape(T, HD) * norm_w * torch.nn.functional.silu(g.reshape(T, HD))).to(out_dtype)
+
+
+def ref_xielu(a, bias, alpha_pos, alpha_neg, out_dtype):
+    z = a.float() + (bias if bias is not None else 0.0)
+    neg = alpha_neg * (torch.expm1(torch.clamp(z, max=0.0)) - z) + 0.5 * z
+    return torch.where(z > 0, alpha_pos * z * z + 0.5 * z, neg).to(out_dtype)
+
+
+def ref_silu_glu(gu, out_dtype):
+    F = gu.shape[1] // 2
+    return (torch.nn.functional.silu(gu[:, :F].float()) * gu[:, F:].float()).to(out_dtype)
 
 
 def ref_limited_glu(gu, limit, out_dtype):
