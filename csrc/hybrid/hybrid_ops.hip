@@ -169,7 +169,7 @@ __global__ void __launch_bounds__(1024) qk_prep_kernel(
     if (is_q && q_scale) k *= q_scale[u];
     // the query factor grows with the logarithm of the position, in steps of qt_every positions
     if (is_q && qt_every > 0) k *= 1.0f + qt_coef * logf((float)((positions[t] + 1) / qt_every) + 1.0f);
-    const float* nw = is_q ? q_w : k_w;                  // a learned weight per channel, or none
+    const float* cw = is_q ? q_w : k_w;                  // a learned weight per channel, or none
     // layout 1: the matrix-core attention kernels' cache (keys chunk-major per block, rt::kc_elem;
     // values transposed [Dv][BS])
     T* dst = is_q ? q + ((size_t)t * H + u) * Dk
@@ -177,7 +177,7 @@ __global__ void __launch_bounds__(1024) qk_prep_kernel(
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int d = lane + 64 * j;
-      if (d < Dk) DT<T>::store(dst + ((!is_q && layout) ? rt::kc_elem(BS, off, d) : d), val[j] * k * (nw ? nw[d] : 1.0f));
+      if (d < Dk) DT<T>::store(dst + ((!is_q && layout) ? rt::kc_elem(BS, off, d) : d), val[j] * k * (cw ? cw[d] : 1.0f));
     }
     if (!is_q) {
       const int g = u - H;
