@@ -448,6 +448,23 @@ def test_other_sizes(tmp_path, run, shape):
     close(got, want, run, shape)
 
 
+@pytest.mark.parametrize("run", RUNS)
+def test_wider_layers(tmp_path, run):
+    """Rows wide enough for several waves per norm workgroup, wkv heads that fill a wave, 64-wide
+    attention heads with a window that crosses many key tiles and pages, eight experts: a prompt in
+    portions (the first long enough for seven scan chunks), then decoded tokens."""
+    layers = [wkv(8, 64, mlp={"kind": "dense", "ff": 1024}, rank=32), att(8, 2, 64, window=200, temp=(0.2, 128), mlp=moe(8, 2, 256))]
+    cfg = make_config(width=512, vocab=331, layers=layers, loop=(0, 2, 2), groups=2)
+    P = make_checkpoint(tmp_path / "m", cfg, seed=21)
+    e = engine_for(tmp_path / "m", run, tokens=1024, block_size=32)
+    t = toks(720, cfg["vocab"], 21)
+    want = forward(cfg, P, t)
+    got = [e.step([("a", t[:450], [0, 199, 200, 201, 449])]), e.step([("a", t[450:452], [0, 1])]),
+           e.step([("a", t[452:700], [0, 247])])] + [e.step([("a", t[i:i + 1], [0])]) for i in range(700, 720)]
+    rows = [0, 199, 200, 201, 449, 450, 451, 452, 699] + list(range(700, 720))
+    close(torch.cat(got), want[rows], run, "wider layers")
+
+
 # ---- portions, decoding, batches ------------------------------------------------------------------
 
 @pytest.mark.parametrize("run", RUNS)
