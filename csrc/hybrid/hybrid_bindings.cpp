@@ -304,7 +304,7 @@ void wkv_scan(torch::Tensor out, torch::Tensor rkvg, torch::Tensor lw, torch::Te
     chk_i32(*chunks, "chunks"); chk_i32(*seq_chunk0, "seq_chunk0", S + 1); chk_f32(*ws, "ws");
     TORCH_CHECK(chunks->dim() == 2 && chunks->size(1) == 2, "wkv_scan: chunks [n, 2]");
     n = chunks->size(0);
-    TORCH_CHECK(ws->numel() >= n * H * (2 * D * D + D), "wkv_scan: workspace too small");
+    TORCH_CHECK(ws->numel() >= n * H * (D * D + D), "wkv_scan: workspace too small");
     ch = chunks->data_ptr<int>(); sc0 = seq_chunk0->data_ptr<int>(); wsp = ws->data_ptr<float>();
   }
   const char* base = static_cast<const char*>(rkvg.data_ptr());
@@ -313,7 +313,7 @@ void wkv_scan(torch::Tensor out, torch::Tensor rkvg, torch::Tensor lw, torch::Te
                            w0.data_ptr<float>(), u.data_ptr<float>(), norm_w.data_ptr<float>(), state.data_ptr<float>(),
                            cu_q.data_ptr<int>(), start_pos.data_ptr<int>(), slots.data_ptr<int>(), S, H, D, (float)eps, ch,
                            n, sc0, wsp, is_bf(rkvg), cur());
-  TORCH_CHECK(rc == 0, "wkv_scan: unsupported shape");
+  TORCH_CHECK(rc == 0, "wkv_scan: unsupported shape (code ", rc, ")");
 }
 
 void xielu(torch::Tensor out, torch::Tensor a, c10::optional<torch::Tensor> bias, double ap, double an) {

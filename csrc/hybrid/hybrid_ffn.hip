@@ -8,8 +8,9 @@
 //                    mixture of gated experts, no host round trip so a graph can hold it):
 //                    hid[t, k, :] = silu(Wg[e] h_t) * (Wu[e] h_t),  e = idx[t, k]
 //                    out[t, :]    = sum_k wt[t, k] * Wd[e] hid[t, k, :]
-//                    One wave per output entry walks a weight row in 16-byte loads against the
-//                    input row staged in LDS as fp32; a row's result does not depend on the others.
+//                    One wave per four output entries walks their weight rows in 16-byte loads (all
+//                    in flight together) against the input row staged in LDS as fp32; a row's
+//                    result does not depend on the others.
 #include "../common.h"
 
 namespace {
@@ -79,79 +80,135 @@ __global__ void __launch_bounds__(64) topk_softmax_kernel(int* __restrict__ idx,
   }
 }
 
-// sum over n entries of w[i] * x[i] for the whole wave; x fp32 in LDS, w a weight row in memory
-template <typename T>
-RT_DEVICE float wave_dot(const T* __restrict__ w, const float* __restrict__ x, int n, int lane);
-
-template <>
-RT_DEVICE float wave_dot<uint16_t>(const uint16_t* __restrict__ w, const float* __restrict__ x, int n, int lane) {
-  float acc = 0.f;
-  if ((n & 7) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0) {
-    for (int c = lane * 8; c < n; c += 512) {
-      const rt::short8 p = *reinterpret_cast<const rt::short8*>(w + c);
+// R dot products at once for the whole wave: rows w, w + rs, ... (the first `ok` of them) against
+// x (fp32 in LDS), n entries each. The R rows' loads of a step are independent, so they are all in
+// flight before the first multiply; x is read once per step for all rows.
+template <int R>
+RT_DEVICE void dot_rows_bf16(const uint16_t* __restrict__ w, size_t rs, int ok, const float* __restrict__ x, int n,
+                             int lane, float* out) {
+  float acc[R];
 #pragma unroll
-      for (int q = 0; q < 8; ++q) acc += rt::bf2f((uint16_t)p[q]) * x[c + q];
+  for (int r = 0; r < R; ++r) acc[r] = 0.f;
+  if ((n & 7) == 0 && (rs & 7) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0) {
+    for (int c = lane * 8; c < n; c += 512) {
+      rt::short8 p[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) p[r] = *reinterpret_cast<const rt::short8*>(w + (size_t)(r < ok ? r : 0) * rs + c);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const float xv = x[c + q];
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[r] += rt::bf2f((uint16_t)p[r][q]) * xv;
+      }
     }
   } else {
-    for (int c = lane; c < n; c += 64) acc += rt::bf2f(w[c]) * x[c];
+    for (int c = lane; c < n; c += 64) {
+      const float xv = x[c];
+#pragma unroll
+      for (int r = 0; r < R; ++r) acc[r] += rt::bf2f(w[(size_t)(r < ok ? r : 0) * rs + c]) * xv;
+    }
   }
-  return rt::wave_sum(acc);
+#pragma unroll
+  for (int r = 0; r < R; ++r) out[r] = rt::wave_sum(acc[r]);
 }
 
-template <>
-RT_DEVICE float wave_dot<float>(const float* __restrict__ w, const float* __restrict__ x, int n, int lane) {
-  float acc = 0.f;
-  if ((n & 3) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0) {
+template <int R>
+RT_DEVICE void dot_rows_f32(const float* __restrict__ w, size_t rs, int ok, const float* __restrict__ x, int n, int lane,
+                            float* out) {
+  float acc[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) acc[r] = 0.f;
+  if ((n & 3) == 0 && (rs & 3) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0) {
     for (int c = lane * 4; c < n; c += 256) {
-      const float4 p = *reinterpret_cast<const float4*>(w + c);
-      acc += p.x * x[c] + p.y * x[c + 1] + p.z * x[c + 2] + p.w * x[c + 3];
+      float4 p[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) p[r] = *reinterpret_cast<const float4*>(w + (size_t)(r < ok ? r : 0) * rs + c);
+      const float x0 = x[c], x1 = x[c + 1], x2 = x[c + 2], x3 = x[c + 3];
+#pragma unroll
+      for (int r = 0; r < R; ++r) acc[r] += p[r].x * x0 + p[r].y * x1 + p[r].z * x2 + p[r].w * x3;
     }
   } else {
-    for (int c = lane; c < n; c += 64) acc += w[c] * x[c];
+    for (int c = lane; c < n; c += 64) {
+      const float xv = x[c];
+#pragma unroll
+      for (int r = 0; r < R; ++r) acc[r] += w[(size_t)(r < ok ? r : 0) * rs + c] * xv;
+    }
   }
-  return rt::wave_sum(acc);
+#pragma unroll
+  for (int r = 0; r < R; ++r) out[r] = rt::wave_sum(acc[r]);
+}
+
+template <int R>
+RT_DEVICE void dot_rows(const uint16_t* w, size_t rs, int ok, const float* x, int n, int lane, float* out) {
+  dot_rows_bf16<R>(w, rs, ok, x, n, lane, out);
+}
+template <int R>
+RT_DEVICE void dot_rows(const float* w, size_t rs, int ok, const float* x, int n, int lane, float* out) {
+  dot_rows_f32<R>(w, rs, ok, x, n, lane, out);
 }
 
 constexpr int kMoeWaves = 4;
+constexpr int kMoeRows = 4;         // output entries a wave computes together
+constexpr int kMoeBlock = kMoeWaves * kMoeRows;
 
-// grid (T * top, blocks over F); wgu [E, 2F, W] = (gate | up) rows of every expert
+// grid (T * top, blocks of kMoeBlock over F); wgu [E, 2F, W] = (gate | up) rows of every expert
 template <typename T>
 __global__ void __launch_bounds__(64 * kMoeWaves) moe_gate_up_kernel(float* __restrict__ hid, const T* __restrict__ h,
                                                                      const T* __restrict__ wgu,
-                                                                     const int* __restrict__ idx, int W, int F, int top,
-                                                                     int per_block) {
+                                                                     const int* __restrict__ idx, int W, int F, int top) {
   extern __shared__ float xs[];
   const int pair = blockIdx.x, t = pair / top;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (int c = threadIdx.x; c < W; c += blockDim.x) xs[c] = DT<T>::load(h + (size_t)t * W + c);
   __syncthreads();
   const T* we = wgu + (size_t)idx[pair] * 2 * F * W;
-  const int f0 = blockIdx.y * per_block, f1 = min(F, f0 + per_block);
-  for (int f = f0 + wave; f < f1; f += kMoeWaves) {
-    const float g = wave_dot<T>(we + (size_t)f * W, xs, W, lane);
-    const float u = wave_dot<T>(we + (size_t)(F + f) * W, xs, W, lane);
-    if (lane == 0) hid[(size_t)pair * F + f] = g * sigm(g) * u;
+  const int f = blockIdx.y * kMoeBlock + wave * kMoeRows;
+  const int ok = min(kMoeRows, F - f);
+  if (ok <= 0) return;
+  float gv[kMoeRows], uv[kMoeRows];
+  dot_rows<kMoeRows>(we + (size_t)f * W, (size_t)W, ok, xs, W, lane, gv);
+  dot_rows<kMoeRows>(we + (size_t)(F + f) * W, (size_t)W, ok, xs, W, lane, uv);
+  if (lane < ok) {
+    float g = 0.f, u = 0.f;
+#pragma unroll
+    for (int r = 0; r < kMoeRows; ++r)
+      if (r == lane) {
+        g = gv[r];
+        u = uv[r];
+      }
+    hid[(size_t)pair * F + f + lane] = g * sigm(g) * u;
   }
 }
 
-// grid (T, blocks over W); wd [E, W, F]
+// grid (T, blocks of kMoeBlock over W); wd [E, W, F]
 template <typename T>
 __global__ void __launch_bounds__(64 * kMoeWaves) moe_down_kernel(T* __restrict__ out, const float* __restrict__ hid,
                                                                   const T* __restrict__ wd, const int* __restrict__ idx,
-                                                                  const float* __restrict__ wt, int W, int F, int top,
-                                                                  int per_block) {
+                                                                  const float* __restrict__ wt, int W, int F, int top) {
   extern __shared__ float xs[];       // [top][F]
   const int t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (int c = threadIdx.x; c < top * F; c += blockDim.x) xs[c] = hid[(size_t)t * top * F + c];
   __syncthreads();
-  const int c0 = blockIdx.y * per_block, c1 = min(W, c0 + per_block);
-  for (int c = c0 + wave; c < c1; c += kMoeWaves) {
-    float acc = 0.f;
-    for (int k = 0; k < top; ++k)
-      acc += wt[(size_t)t * top + k] *
-             wave_dot<T>(wd + ((size_t)idx[(size_t)t * top + k] * W + c) * F, xs + (size_t)k * F, F, lane);
-    if (lane == 0) DT<T>::store(out + (size_t)t * W + c, acc);
+  const int c0 = blockIdx.y * kMoeBlock + wave * kMoeRows;
+  const int ok = min(kMoeRows, W - c0);
+  if (ok <= 0) return;
+  float acc[kMoeRows];
+#pragma unroll
+  for (int r = 0; r < kMoeRows; ++r) acc[r] = 0.f;
+  for (int k = 0; k < top; ++k) {
+    float d[kMoeRows];
+    dot_rows<kMoeRows>(wd + ((size_t)idx[(size_t)t * top + k] * W + c0) * F, (size_t)F, ok, xs + (size_t)k * F, F, lane, d);
+    const float c = wt[(size_t)t * top + k];
+#pragma unroll
+    for (int r = 0; r < kMoeRows; ++r) acc[r] += c * d[r];
+  }
+  if (lane < ok) {
+    float v = 0.f;
+#pragma unroll
+    for (int r = 0; r < kMoeRows; ++r)
+      if (r == lane) v = acc[r];
+    DT<T>::store(out + (size_t)t * W + c0 + lane, v);
   }
 }
 
@@ -186,8 +243,8 @@ int launch_moe_rows(void* out, float* hid, const void* h, const void* wgu, const
   if (T <= 0) return 0;
   const size_t shm1 = sizeof(float) * (size_t)W, shm2 = sizeof(float) * (size_t)top * F;
   if (shm1 > 150 * 1024 || shm2 > 150 * 1024) return -1;
-  // about 16 output entries per wave: enough workgroups to fill the chip from a handful of rows
-  const int pb = 16 * kMoeWaves;
+  // four output entries per wave: enough workgroups to fill the chip from a handful of rows
+  const int pb = kMoeBlock;
   const dim3 g1(T * top, (F + pb - 1) / pb), g2(T, (W + pb - 1) / pb);
 #define RT_MOE(TT)                                                                                                     \
   do {                                                                                                                 \
@@ -199,8 +256,8 @@ int launch_moe_rows(void* out, float* hid, const void* h, const void* wgu, const
     if (shm2 > 48 * 1024 &&                                                                                            \
         hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm2) != hipSuccess)     \
       return -2;                                                                                                       \
-    k1<<<g1, 64 * kMoeWaves, shm1, stream>>>(hid, (const TT*)h, (const TT*)wgu, idx, W, F, top, pb);                   \
-    k2<<<g2, 64 * kMoeWaves, shm2, stream>>>((TT*)out, hid, (const TT*)wd, idx, wt, W, F, top, pb);                    \
+    k1<<<g1, 64 * kMoeWaves, shm1, stream>>>(hid, (const TT*)h, (const TT*)wgu, idx, W, F, top);                       \
+    k2<<<g2, 64 * kMoeWaves, shm2, stream>>>((TT*)out, hid, (const TT*)wd, idx, wt, W, F, top);                        \
   } while (0)
   if (bf) RT_MOE(uint16_t); else RT_MOE(float);
 #undef RT_MOE

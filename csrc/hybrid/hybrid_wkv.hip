@@ -8,23 +8,30 @@
 //     out_t[j]   = o_t[j] / rms_j(o_t) * norm_w[j] * silu(g_t[j])
 //
 // One workgroup per (sequence, head); thread j owns value column j and keeps S[.][j] in registers
-// (DB = the power of two >= D, at least 64; rows i >= D are never touched). r, k and the decay of a
-// token are staged in LDS (two buffers, one barrier a token) and read by every thread.
+// (DB = the power of two >= D, at least 64; rows i >= D are never touched). The rows of a span are
+// taken in blocks of up to SB tokens: every thread first copies its column of r, k, v, the gate and
+// the decay of the whole block to LDS (independent loads, all in flight together), then the
+// recurrence runs over the block reading LDS only — no global load and, for heads of up to 64
+// columns (one wave), no barrier inside the token loop.
 //
 // Long spans run in three launches over chunks of kWkvChunk rows, like the minGRU scan: (A) every
 // chunk alone from S = 0: its end state E and its decay product Pd[i]; (B) per (sequence, head),
-// chunk by chunk: the state each chunk starts from (carry = Pd * carry + E) and the sequence's new
-// state; (C) every chunk again from its true start state, writing the outputs. No division by a
-// decay product anywhere, so small decays are harmless.
+// chunk by chunk: the state each chunk starts from (carry = Pd * carry + E, written over E) and the
+// sequence's new state; (C) every chunk again from its true start state, writing the outputs. No
+// division by a decay product anywhere, so small decays are harmless.
 #include "../common.h"
 
 namespace {
 
 using rt::DT;
 
-constexpr int kWkvChunk = 64;
+constexpr int kWkvChunk = 32;
 
 RT_DEVICE float sigm(float v) { return 1.0f / (1.0f + expf(-v)); }
+
+// tokens staged at a time: 5 arrays of SB x DB floats (40 KB at DB = 64, 80 KB at 128 and 256)
+template <int DB> constexpr int stage_rows() { return DB <= 64 ? 32 : DB <= 128 ? 32 : 16; }
+template <int DB> constexpr size_t wkv_lds_bytes() { return sizeof(float) * ((size_t)5 * stage_rows<DB>() * DB + DB + 8); }
 
 // MODE 0: whole spans, state in and out of the slots. MODE 1: phase A. MODE 3: phase C.
 template <typename T, int DB, int MODE>
@@ -33,9 +40,16 @@ __global__ void __launch_bounds__(DB) wkv_scan_kernel(
     const T* __restrict__ g, const T* __restrict__ lw, int stride, int lw_stride, const float* __restrict__ w0,
     const float* __restrict__ u, const float* __restrict__ norm_w, float* __restrict__ state,
     const int* __restrict__ cu_q, const int* __restrict__ start_pos, const int* __restrict__ slots,
-    const int* __restrict__ chunks, float* __restrict__ ws_e, float* __restrict__ ws_p,
-    const float* __restrict__ ws_in, int H, int D, float eps) {
-  __shared__ float sr[2][DB], sk[2][DB], sw[2][DB], su[DB], red[2][DB / 64];
+    const int* __restrict__ chunks, float* __restrict__ ws_e, float* __restrict__ ws_p, int H, int D, float eps) {
+  constexpr int SB = stage_rows<DB>();
+  extern __shared__ float lds[];
+  float* sr = lds;                  // [SB][DB] each
+  float* sk = sr + SB * DB;
+  float* sw = sk + SB * DB;
+  float* sv = sw + SB * DB;
+  float* sg = sv + SB * DB;
+  float* su = sg + SB * DB;         // [DB]
+  float* red = su + DB;             // [2][4]
   const int j = threadIdx.x, lane = j & 63, wid = j >> 6;
   const int h = blockIdx.y;
   int s, r0, r1;
@@ -59,7 +73,7 @@ __global__ void __launch_bounds__(DB) wkv_scan_kernel(
 #pragma unroll
     for (int i = 0; i < DB; ++i) S[i] = (keep && on && i < D) ? st[(size_t)i * D + j] : 0.f;
   } else if (MODE == 3) {
-    const float* in = ws_in + ((size_t)blockIdx.x * H + h) * DD;
+    const float* in = ws_e + ((size_t)blockIdx.x * H + h) * DD;      // phase B left the start state here
 #pragma unroll
     for (int i = 0; i < DB; ++i) S[i] = (on && i < D) ? in[(size_t)i * D + j] : 0.f;
   } else {
@@ -70,39 +84,53 @@ __global__ void __launch_bounds__(DB) wkv_scan_kernel(
   su[j] = on ? u[col] : 0.f;
   const float w0j = on ? w0[col] : 0.f, nwj = on && MODE != 1 ? norm_w[col] : 0.f;
   float pd = 1.f;
-  for (int t = r0; t < r1; ++t) {
-    const int b = (t - r0) & 1;
-    float vj = 0.f, gj = 0.f;
+  for (int t0 = r0; t0 < r1; t0 += SB) {
+    const int n = min(SB, r1 - t0);
+    __syncthreads();        // the previous block's readers are done
     if (on) {
-      const size_t at = (size_t)t * stride + col;
-      const float dec = expf(-expf(DT<T>::load(lw + (size_t)t * lw_stride + col) + w0j));
-      sr[b][j] = MODE == 1 ? 0.f : DT<T>::load(r + at);
-      sk[b][j] = DT<T>::load(k + at);
-      sw[b][j] = dec;
-      vj = DT<T>::load(v + at);
-      if (MODE != 1) gj = DT<T>::load(g + at);
-      pd *= dec;
-    }
-    __syncthreads();        // the token's r, k, decay are staged (the other buffer's readers are done)
-    float acc = 0.f;
-#pragma unroll
-    for (int i = 0; i < DB; ++i) {
-      if (i < D) {
-        const float kv = sk[b][i] * vj;
-        if (MODE != 1) acc += sr[b][i] * (S[i] + su[i] * kv);
-        S[i] = sw[b][i] * S[i] + kv;
+#pragma unroll 8
+      for (int tt = 0; tt < n; ++tt) {
+        const size_t at = (size_t)(t0 + tt) * stride + col;
+        const float dec = expf(-expf(DT<T>::load(lw + (size_t)(t0 + tt) * lw_stride + col) + w0j));
+        sk[tt * DB + j] = DT<T>::load(k + at);
+        sv[tt * DB + j] = DT<T>::load(v + at);
+        sw[tt * DB + j] = dec;
+        if (MODE != 1) {
+          sr[tt * DB + j] = DT<T>::load(r + at);
+          sg[tt * DB + j] = DT<T>::load(g + at);
+        }
+        pd *= dec;
       }
     }
-    if (MODE != 1) {
-      float ss = rt::wave_sum(on ? acc * acc : 0.f);
-      if (DB > 64) {
-        if (lane == 0) red[b][wid] = ss;
-        __syncthreads();
-        ss = 0.f;
+    __syncthreads();        // the block's r, k, decay are staged
+    for (int tt = 0; tt < n; ++tt) {
+      const float* kr = sk + tt * DB;
+      const float* rr = sr + tt * DB;
+      const float* wr = sw + tt * DB;
+      const float vj = sv[tt * DB + j];
+      float acc = 0.f;
 #pragma unroll
-        for (int q = 0; q < DB / 64; ++q) ss += red[b][q];
+      for (int i = 0; i < DB; ++i) {
+        if (i < D) {
+          const float kv = kr[i] * vj;
+          if (MODE != 1) acc += rr[i] * (S[i] + su[i] * kv);
+          S[i] = wr[i] * S[i] + kv;
+        }
       }
-      if (on) DT<T>::store(out + (size_t)t * stride + col, acc / sqrtf(ss / (float)D + eps) * nwj * (gj * sigm(gj)));
+      if (MODE != 1) {
+        float ss = rt::wave_sum(on ? acc * acc : 0.f);
+        if (DB > 64) {
+          const int b = tt & 1;
+          if (lane == 0) red[b * 4 + wid] = ss;
+          __syncthreads();
+          ss = 0.f;
+#pragma unroll
+          for (int q = 0; q < DB / 64; ++q) ss += red[b * 4 + q];
+        }
+        const float gj = sg[tt * DB + j];
+        if (on)
+          DT<T>::store(out + (size_t)(t0 + tt) * stride + col, acc / sqrtf(ss / (float)D + eps) * nwj * (gj * sigm(gj)));
+      }
     }
   }
   if (!on) return;
@@ -119,10 +147,10 @@ __global__ void __launch_bounds__(DB) wkv_scan_kernel(
   }
 }
 
-// phase B: grid (sequences, heads, row blocks of the state), thread = one (i, j) entry of S
-__global__ void __launch_bounds__(256) wkv_carry_kernel(const float* __restrict__ ws_e, const float* __restrict__ ws_p,
-                                                        float* __restrict__ ws_in, float* __restrict__ state,
-                                                        const int* __restrict__ seq_chunk0,
+// phase B: grid (sequences, heads, row blocks of the state), thread = one (i, j) entry of S; every
+// chunk's end state in ws_e is replaced by the state the chunk starts from
+__global__ void __launch_bounds__(256) wkv_carry_kernel(float* __restrict__ ws_e, const float* __restrict__ ws_p,
+                                                        float* __restrict__ state, const int* __restrict__ seq_chunk0,
                                                         const int* __restrict__ start_pos, const int* __restrict__ slots,
                                                         int H, int D) {
   const int s = blockIdx.x, h = blockIdx.y;
@@ -135,10 +163,40 @@ __global__ void __launch_bounds__(256) wkv_carry_kernel(const float* __restrict_
   float S = start_pos[s] > 0 ? *st : 0.f;
   for (int c = k0; c < k1; ++c) {
     const size_t at = (size_t)c * H + h;
-    ws_in[at * DD + e] = S;
-    S = ws_p[at * D + i] * S + ws_e[at * DD + e];
+    const float E = ws_e[at * DD + e];
+    ws_e[at * DD + e] = S;
+    S = ws_p[at * D + i] * S + E;
   }
   *st = S;
+}
+
+template <typename T, int DB, int MODE>
+int launch_one(dim3 grid, hipStream_t stream, T* out, const T* r, const T* k, const T* v, const T* g, const T* lw,
+               int stride, int lw_stride, const float* w0, const float* u, const float* norm_w, float* state,
+               const int* cu_q, const int* start_pos, const int* slots, const int* chunks, float* ws_e, float* ws_p, int H,
+               int D, float eps) {
+  auto kern = wkv_scan_kernel<T, DB, MODE>;
+  const size_t shm = wkv_lds_bytes<DB>();
+  if (shm > 48 * 1024 &&
+      hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm) != hipSuccess)
+    return -2;
+  kern<<<grid, DB, shm, stream>>>(out, r, k, v, g, lw, stride, lw_stride, w0, u, norm_w, state, cu_q, start_pos, slots,
+                                  chunks, ws_e, ws_p, H, D, eps);
+  return 0;
+}
+
+template <typename T, int MODE>
+int launch_mode(int db, dim3 grid, hipStream_t stream, void* out, const void* r, const void* k, const void* v,
+                const void* g, const void* lw, int stride, int lw_stride, const float* w0, const float* u,
+                const float* norm_w, float* state, const int* cu_q, const int* start_pos, const int* slots,
+                const int* chunks, float* ws_e, float* ws_p, int H, int D, float eps) {
+#define RT_WKV(DBV)                                                                                                   \
+  launch_one<T, DBV, MODE>(grid, stream, (T*)out, (const T*)r, (const T*)k, (const T*)v, (const T*)g, (const T*)lw,   \
+                           stride, lw_stride, w0, u, norm_w, state, cu_q, start_pos, slots, chunks, ws_e, ws_p, H, D, eps)
+  if (db == 64) return RT_WKV(64);
+  if (db == 128) return RT_WKV(128);
+  return RT_WKV(256);
+#undef RT_WKV
 }
 
 }  // namespace
@@ -146,7 +204,7 @@ __global__ void __launch_bounds__(256) wkv_carry_kernel(const float* __restrict_
 int wkv_scan_chunk() { return kWkvChunk; }
 
 // chunks == nullptr: one launch over whole spans (grid S x H). Otherwise the three launches over
-// `n_chunks` chunks; ws holds n_chunks * H * (2 * D * D + D) floats.
+// `n_chunks` chunks; ws holds n_chunks * H * (D * D + D) floats.
 int launch_wkv_scan(void* out, const void* r, const void* k, const void* v, const void* g, const void* lw, int stride,
                     int lw_stride, const float* w0, const float* u, const float* norm_w, float* state, const int* cu_q,
                     const int* start_pos, const int* slots, int S, int H, int D, float eps, const int* chunks,
@@ -156,33 +214,18 @@ int launch_wkv_scan(void* out, const void* r, const void* k, const void* v, cons
   const int db = D <= 64 ? 64 : D <= 128 ? 128 : 256;
   const size_t DD = (size_t)D * D;
   float* ws_e = ws;
-  float* ws_in = ws ? ws + (size_t)n_chunks * H * DD : nullptr;
-  float* ws_p = ws ? ws + 2 * (size_t)n_chunks * H * DD : nullptr;
-#define RT_WKV(TT, DBV, MODE, GRID)                                                                                  \
-  wkv_scan_kernel<TT, DBV, MODE><<<GRID, DBV, 0, stream>>>((TT*)out, (const TT*)r, (const TT*)k, (const TT*)v,       \
-                                                           (const TT*)g, (const TT*)lw, stride, lw_stride, w0, u,    \
-                                                           norm_w, state, cu_q, start_pos, slots, chunks, ws_e,      \
-                                                           ws_p, ws_in, H, D, eps)
-#define RT_WKV_T(DBV, MODE, GRID)                                                                                    \
-  do {                                                                                                               \
-    if (bf) RT_WKV(uint16_t, DBV, MODE, GRID); else RT_WKV(float, DBV, MODE, GRID);                                  \
-  } while (0)
-#define RT_WKV_D(MODE, GRID)                                                                                         \
-  do {                                                                                                               \
-    if (db == 64) RT_WKV_T(64, MODE, GRID); else if (db == 128) RT_WKV_T(128, MODE, GRID);                           \
-    else RT_WKV_T(256, MODE, GRID);                                                                                  \
-  } while (0)
-  if (chunks == nullptr) {
-    RT_WKV_D(0, dim3(S, H));
-    return 0;
-  }
+  float* ws_p = ws ? ws + (size_t)n_chunks * H * DD : nullptr;
+#define RT_WKV_M(MODE, GRID)                                                                                          \
+  (bf ? launch_mode<uint16_t, MODE>(db, GRID, stream, out, r, k, v, g, lw, stride, lw_stride, w0, u, norm_w, state,   \
+                                    cu_q, start_pos, slots, chunks, ws_e, ws_p, H, D, eps)                            \
+      : launch_mode<float, MODE>(db, GRID, stream, out, r, k, v, g, lw, stride, lw_stride, w0, u, norm_w, state, cu_q, \
+                                 start_pos, slots, chunks, ws_e, ws_p, H, D, eps))
+  if (chunks == nullptr) return RT_WKV_M(0, dim3(S, H));
   if (n_chunks <= 0) return 0;
-  RT_WKV_D(1, dim3(n_chunks, H));
-  wkv_carry_kernel<<<dim3(S, H, (unsigned)((DD + 255) / 256)), 256, 0, stream>>>(ws_e, ws_p, ws_in, state, seq_chunk0,
-                                                                                 start_pos, slots, H, D);
-  RT_WKV_D(3, dim3(n_chunks, H));
-#undef RT_WKV
-#undef RT_WKV_T
-#undef RT_WKV_D
-  return 0;
+  int rc = RT_WKV_M(1, dim3(n_chunks, H));
+  if (rc) return rc;
+  wkv_carry_kernel<<<dim3(S, H, (unsigned)((DD + 255) / 256)), 256, 0, stream>>>(ws_e, ws_p, state, seq_chunk0, start_pos,
+                                                                                 slots, H, D);
+  return RT_WKV_M(3, dim3(n_chunks, H));
+#undef RT_WKV_M
 }

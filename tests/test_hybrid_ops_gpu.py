@@ -288,7 +288,7 @@ def test_wkv_scan(dt, H, D):
         got = Hy.wkv_scan(*gpu(rkvg, lw, w0, u, nw), 1e-5, *gpu(st_g, cu, sp, slots), dt, chunks=chunks)
         torch.testing.assert_close(got.float().cpu(), want, **t)
         torch.testing.assert_close(st_g.cpu(), st_c, rtol=1e-3, atol=1e-4)
-    assert Hy.wkv_chunks(cu, DEV)[1].tolist() == [0, 1, 2, 3, 6] and Hy.wkv_chunks(torch.tensor([0, 128, 130]), DEV) is None
+    assert Hy.wkv_chunks(cu, DEV)[1].tolist() == [0, 2, 3, 4, 9] and Hy.wkv_chunks(torch.tensor([0, 64, 66]), DEV) is None
 
 
 @pytest.mark.parametrize("dt", DTYPES)

@@ -511,11 +511,12 @@ PRESETS.update({
 PRESETS.update({
     # Retuvik (wkv time mixing with a per-token decay, windowed attention with a distance penalty,
     # xIELU and mixture-of-experts feed-forwards, grouped RMS norms), random-init sizes: a test-sized
-    # stack with a looped middle, and stacks whose layers have the shapes of 1B / 3B / 8B-class Llama
-    # models (every third layer attention, every fourth feed-forward a mixture of 8 experts, 2 per token)
+    # stack with a looped middle, and stacks whose layers have the shapes of 0.5B (Qwen2.5) / 1B / 3B /
+    # 8B-class Llama models (every third layer attention, every fourth feed-forward a mixture of 8 experts, 2 per token)
     "tiny-retuvik": retuvik_config("tiny-retuvik", 4, 128, 4, 2, 32, 256, 32000, attention_every=2, wkv_dim=32,
                                    decay_rank=16, window=24, moe_every=2, experts=6, top=2, expert_ff=64,
                                    loop=(1, 3, 2)),
+    "retuvik-0.5b": retuvik_config("retuvik-0.5b", 24, 896, 14, 2, 64, 4864, 151936, moe_every=4),   # Qwen2.5-0.5B's sizes
     "retuvik-1b": retuvik_config("retuvik-1b", 16, 2048, 32, 8, 64, 8192, 128256, moe_every=4),
     "retuvik-3b": retuvik_config("retuvik-3b", 28, 3072, 24, 8, 128, 8192, 128256, moe_every=4),
     "retuvik-8b": retuvik_config("retuvik-8b", 32, 4096, 32, 8, 128, 14336, 128256, moe_every=4),

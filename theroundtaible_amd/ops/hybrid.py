@@ -263,7 +263,7 @@ def limited_glu(gu, limit: float, out_dtype) -> torch.Tensor:
 
 # ---- wkv ------------------------------------------------------------------------------------------
 
-WKV_CHUNK = 64           # rows per chunk of the chunked wkv scan (csrc/hybrid/hybrid_wkv.hip kWkvChunk)
+WKV_CHUNK = 32           # rows per chunk of the chunked wkv scan (csrc/hybrid/hybrid_wkv.hip kWkvChunk)
 
 
 def wkv_chunks(cu_q: torch.Tensor, device=None, min_rows: int = 2 * WKV_CHUNK):
@@ -294,7 +294,7 @@ def wkv_scan(rkvg, lw, w0, u, norm_w, eps, state, cu_q, start_pos, slots, out_dt
         out = torch.empty(rkvg.shape[1], rkvg.shape[2], dtype=out_dtype, device=rkvg.device)
         if chunks is not None:
             H, D = u.shape
-            ws = torch.empty(chunks[0].shape[0] * H * (2 * D * D + D), dtype=torch.float32, device=rkvg.device)
+            ws = torch.empty(chunks[0].shape[0] * H * (D * D + D), dtype=torch.float32, device=rkvg.device)
             native().wkv_scan(out, rkvg, lw, w0, u, norm_w, float(eps), state, cu_q, start_pos, slots, chunks[0], chunks[1], ws)
         else:
             native().wkv_scan(out, rkvg, lw, w0, u, norm_w, float(eps), state, cu_q, start_pos, slots)
