@@ -2,6 +2,7 @@
 // per-head score multiplier, for any head sizes up to 256 (fp32 FMA form; bf16 or fp32 tensors).
 //
 //   K cache [num_blocks, G, BS, Dk], V cache [num_blocks, G, BS, Dv], q [T, H, Dk], out [T, H * Dv]
+//   (layout 1: the matrix-core kernels' cache — keys chunk-major per block, V [num_blocks, G, Dv, BS])
 //   score(i, j) = q_i . k_j * scale * temp[h] - slopes[h] * (i - j), j <= position(i),
 //                 and i - j < window when a window is given (tiles wholly ahead of it are skipped)
 //   weight_j   = exp(s_j) / (sink + sum_j exp(s_j))        (sink: a key of score 0 without a value)
@@ -36,7 +37,7 @@ __global__ void __launch_bounds__(256) gqa_attention_kernel(
     const int* __restrict__ tiles, const float* __restrict__ temp, float* __restrict__ part_o,
     float* __restrict__ part_ml, int H, int G, int Dk, int Dv, int BS, int max_blocks, int R, int KT, int hchunks,
     float scale, float sink, int window, const float* __restrict__ slopes, const T* __restrict__ gate,
-    int gate_stride) {
+    int gate_stride, int layout) {
   extern __shared__ float lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int seq = tiles[2 * blockIdx.x], row0 = tiles[2 * blockIdx.x + 1];
@@ -88,14 +89,18 @@ __global__ void __launch_bounds__(256) gqa_attention_kernel(
       const int j = i / Dk, d = i - j * Dk;
       const int key = kb + j;
       float v = 0.f;
-      if (key < kend) v = DT<T>::load(kc + (((size_t)bt[key / BS] * G + g) * BS + key % BS) * Dk + d);
+      // layout 1: the cache of the matrix-core kernels (keys chunk-major per block, values [Dv][BS])
+      if (key < kend)
+        v = DT<T>::load(kc + ((size_t)bt[key / BS] * G + g) * BS * Dk +
+                        (layout ? rt::kc_elem(BS, key % BS, d) : (key % BS) * Dk + d));
       ks[j * (Dk + 1) + d] = v;
     }
     for (int i = threadIdx.x; i < KT * Dv; i += blockDim.x) {
       const int j = i / Dv, d = i - j * Dv;
       const int key = kb + j;
       float v = 0.f;
-      if (key < kend) v = DT<T>::load(vc + (((size_t)bt[key / BS] * G + g) * BS + key % BS) * Dv + d);
+      if (key < kend)
+        v = DT<T>::load(vc + ((size_t)bt[key / BS] * G + g) * BS * Dv + (layout ? d * BS + key % BS : (key % BS) * Dv + d));
       vs[i] = v;
     }
     __syncthreads();
@@ -215,7 +220,7 @@ int launch_gqa_attention(void* out, const void* q, const void* kc, const void* v
                          const int* cu_q, const int* start_pos, const int* tiles, int n_tiles, const float* temp,
                          float* part_o, float* part_ml, int T, int H, int G, int Dk, int Dv, int BS, int max_blocks,
                          int rows, int num_splits, float scale, float sink, int window, const float* slopes,
-                         const void* gate, int gate_stride, bool bf, hipStream_t stream) {
+                         const void* gate, int gate_stride, int layout, bool bf, hipStream_t stream) {
   if (n_tiles <= 0 || T <= 0) return 0;
   const int KT = gqa_key_tile(Dk, Dv);
   if (KT == 0 || Dv > 256 || Dk > 256 || H % G) return -1;
@@ -239,7 +244,7 @@ int launch_gqa_attention(void* out, const void* q, const void* kc, const void* v
       return -3;                                                                                                     \
     kern<<<grid, 256, shm, stream>>>((TT*)out, (const TT*)q, (const TT*)kc, (const TT*)vc, block_tables, cu_q,      \
                                      start_pos, tiles, temp, part_o, part_ml, H, G, Dk, Dv, BS, max_blocks, rows,   \
-                                     KT, hchunks, scale, sink, window, slopes, (const TT*)gate, gate_stride);        \
+                                     KT, hchunks, scale, sink, window, slopes, (const TT*)gate, gate_stride, layout); \
   } while (0)
   if (bf) {
     if (dvl == 1) RT_GQA(uint16_t, 1); else if (dvl == 2) RT_GQA(uint16_t, 2); else RT_GQA(uint16_t, 4);

@@ -35,7 +35,7 @@ int launch_gqa_attention(void* out, const void* q, const void* kc, const void* v
                          const int* cu_q, const int* start_pos, const int* tiles, int n_tiles, const float* temp,
                          float* part_o, float* part_ml, int T, int H, int G, int Dk, int Dv, int BS, int max_blocks,
                          int rows, int num_splits, float scale, float sink, int window, const float* slopes,
-                         const void* gate, int gate_stride, bool bf, hipStream_t stream);
+                         const void* gate, int gate_stride, int layout, bool bf, hipStream_t stream);
 int wkv_scan_chunk();
 int launch_wkv_scan(void* out, const void* r, const void* k, const void* v, const void* g, const void* lw, int stride,
                     int lw_stride, const float* w0, const float* u, const float* norm_w, float* state, const int* cu_q,
@@ -165,15 +165,17 @@ void gqa_attention(torch::Tensor out, torch::Tensor q, torch::Tensor kc, torch::
                    torch::Tensor cu_q, torch::Tensor start_pos, torch::Tensor tiles, c10::optional<torch::Tensor> temp,
                    double scale, double sink, int64_t rows, int64_t num_splits, c10::optional<torch::Tensor> part_o,
                    c10::optional<torch::Tensor> part_ml, int64_t window, c10::optional<torch::Tensor> slopes,
-                   c10::optional<torch::Tensor> gate, int64_t gate_off) {
+                   c10::optional<torch::Tensor> gate, int64_t gate_off, int64_t layout) {
   chk_act(out, "out"); chk_act(q, "q"); chk_act(kc, "k_cache"); chk_act(vc, "v_cache");
   TORCH_CHECK(out.scalar_type() == q.scalar_type() && kc.scalar_type() == q.scalar_type() &&
               vc.scalar_type() == q.scalar_type(), "gqa_attention: one dtype for q, the cache and out");
   TORCH_CHECK(q.dim() == 3 && kc.dim() == 4 && vc.dim() == 4 && out.dim() == 2, "gqa_attention: ranks");
   const int64_t T = q.size(0), H = q.size(1), Dk = q.size(2);
-  const int64_t G = kc.size(1), BS = kc.size(2), Dv = vc.size(3);
-  TORCH_CHECK(kc.size(3) == Dk && vc.size(0) == kc.size(0) && vc.size(1) == G && vc.size(2) == BS && H % G == 0,
-              "gqa_attention: cache shapes");
+  TORCH_CHECK(layout == 0 || layout == 1, "gqa_attention: layout 0 (rows) or 1 (matrix-core kernels)");
+  const int64_t G = kc.size(1), BS = kc.size(2), Dv = vc.size(layout ? 2 : 3);
+  TORCH_CHECK(kc.size(3) == Dk && vc.size(0) == kc.size(0) && vc.size(1) == G && vc.size(layout ? 3 : 2) == BS &&
+              H % G == 0, "gqa_attention: cache shapes");
+  TORCH_CHECK(layout == 0 || Dk % 32 == 0, "gqa_attention: the matrix-core key layout needs dim % 32 == 0");
   TORCH_CHECK(out.size(0) == T && out.size(1) == H * Dv, "gqa_attention: out [T, H * Dv]");
   chk_i32(block_tables, "block_tables"); chk_i32(cu_q, "cu_q"); chk_i32(start_pos, "start_pos", cu_q.numel() - 1);
   chk_i32(tiles, "tiles");
@@ -211,7 +213,7 @@ void gqa_attention(torch::Tensor out, torch::Tensor q, torch::Tensor kc, torch::
   int rc = launch_gqa_attention(out.data_ptr(), q.data_ptr(), kc.data_ptr(), vc.data_ptr(), block_tables.data_ptr<int>(),
                                 cu_q.data_ptr<int>(), start_pos.data_ptr<int>(), tiles.data_ptr<int>(), tiles.size(0), tp,
                                 po, pml, T, H, G, Dk, Dv, BS, block_tables.size(1), rows, num_splits, (float)scale,
-                                (float)sink, (int)window, sl, gp, (int)gstride, is_bf(q), cur());
+                                (float)sink, (int)window, sl, gp, (int)gstride, (int)layout, is_bf(q), cur());
   TORCH_CHECK(rc == 0, "gqa_attention: unsupported shape (code ", rc, ": -1 head sizes beyond 256 or the LDS tile, "
               "-2 rows per tile, -3 LDS size refused)");
 }
@@ -373,7 +375,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("gqa_attention", &gqa_attention, py::arg("out"), py::arg("q"), py::arg("kc"), py::arg("vc"),
         py::arg("block_tables"), py::arg("cu_q"), py::arg("start_pos"), py::arg("tiles"), py::arg("temp"), py::arg("scale"),
         py::arg("sink"), py::arg("rows"), py::arg("num_splits"), py::arg("part_o"), py::arg("part_ml"),
-        py::arg("window") = 0, py::arg("slopes") = py::none(), py::arg("gate") = py::none(), py::arg("gate_off") = 0);
+        py::arg("window") = 0, py::arg("slopes") = py::none(), py::arg("gate") = py::none(), py::arg("gate_off") = 0,
+        py::arg("layout") = 0);
   m.def("mingru_scan", &mingru_scan, py::arg("out"), py::arg("proj"), py::arg("z_off"), py::arg("x_off"), py::arg("g_off"),
         py::arg("bz"), py::arg("bx"), py::arg("state"), py::arg("cu_q"), py::arg("start_pos"), py::arg("slots"),
         py::arg("chunks") = py::none(), py::arg("seq_chunk0") = py::none(), py::arg("ws") = py::none());

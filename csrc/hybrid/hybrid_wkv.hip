@@ -101,6 +101,18 @@ __global__ void __launch_bounds__(DB) wkv_scan_kernel(
         }
         pd *= dec;
       }
+    } else {
+      // key channels past D: zeros, so the token loop runs over all DB rows without a test and
+      // those rows of S stay zero
+      for (int tt = 0; tt < n; ++tt) {
+        sk[tt * DB + j] = 0.f;
+        sw[tt * DB + j] = 0.f;
+        sv[tt * DB + j] = 0.f;
+        if (MODE != 1) {
+          sr[tt * DB + j] = 0.f;
+          sg[tt * DB + j] = 0.f;
+        }
+      }
     }
     __syncthreads();        // the block's r, k, decay are staged
     for (int tt = 0; tt < n; ++tt) {
@@ -108,15 +120,14 @@ __global__ void __launch_bounds__(DB) wkv_scan_kernel(
       const float* rr = sr + tt * DB;
       const float* wr = sw + tt * DB;
       const float vj = sv[tt * DB + j];
-      float acc = 0.f;
+      float a4[4] = {0.f, 0.f, 0.f, 0.f};     // four partial sums: no 64-long dependent chain
 #pragma unroll
       for (int i = 0; i < DB; ++i) {
-        if (i < D) {
-          const float kv = kr[i] * vj;
-          if (MODE != 1) acc += rr[i] * (S[i] + su[i] * kv);
-          S[i] = wr[i] * S[i] + kv;
-        }
+        const float kv = kr[i] * vj;
+        if (MODE != 1) a4[i & 3] += rr[i] * (S[i] + su[i] * kv);
+        S[i] = wr[i] * S[i] + kv;
       }
+      const float acc = (a4[0] + a4[1]) + (a4[2] + a4[3]);
       if (MODE != 1) {
         float ss = rt::wave_sum(on ? acc * acc : 0.f);
         if (DB > 64) {

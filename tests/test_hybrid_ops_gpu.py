@@ -323,3 +323,65 @@ def test_feed_forward_kernels(dt):
     want = Hy.moe_experts(h2.float(), idx.cpu(), wt.cpu(), w2.float(), d2.float(), torch.float32)
     got = Hy.moe_experts(*gpu(h2, idx, wt, w2, d2), dt, by_row=True)
     torch.testing.assert_close(got.float().cpu(), want, **tol(dt))
+
+
+@pytest.mark.parametrize("shape", [(4, 2, 64, 11), (8, 1, 64, 150), (7, 7, 128, 40), (16, 2, 128, 300), (3, 1, 128, 33)])
+def test_matrix_core_prefill_with_window_and_penalty(shape):
+    """The framework's bf16 matrix-core prompt attention in its window / penalty variant, and the
+    any-size kernel reading the same cache layout (decode rows of such a layer), against the
+    statement on a cache of plain rows filled from the same projections."""
+    from theroundtaible_amd import ops
+    if not ops.native_available():
+        pytest.skip("main extension not built")
+    H, G, D, window = shape
+    dt, BS = torch.bfloat16, 32
+    g = torch.Generator().manual_seed(H * D + window)
+    lens, starts = [70, 1, 2, 133], [0, 130, 63, 5]
+    cu, _, pos, sp = spans(lens, starts)
+    T = sum(lens)
+    ctx = [s + n for s, n in zip(starts, lens)]
+    nblk = [(c + BS - 1) // BS for c in ctx]
+    nb = sum(nblk) + 2
+    perm = torch.randperm(nb, generator=g).tolist()
+    bt = torch.zeros(len(lens), max(nblk), dtype=torch.int32)
+    for s, n in enumerate(nblk):
+        bt[s, :n] = torch.tensor([perm.pop() for _ in range(n)])
+    spec = GroupedAttentionSpec(H, G, D, D, 1.0, value_norm=True)
+    slopes = torch.tensor([2.0 ** (-8.0 * (a + 1) / H) for a in range(H)])
+    # every sequence's whole context goes through qk_prep once per layout (keys of the span rows and before)
+    caches = {}
+    for layout in (False, True):
+        kc = torch.zeros(nb, G, BS, D, dtype=dt, device=DEV)
+        vc = torch.zeros((nb, G, D, BS) if layout else (nb, G, BS, D), dtype=dt, device=DEV)
+        gq = torch.Generator().manual_seed(7)
+        qs = []
+        for s in range(len(lens)):
+            n = ctx[s]
+            proj = (torch.randn(n, (H + 2 * G) * D, generator=gq) * 0.7).to(dt).to(DEV)
+            slots = torch.tensor([int(bt[s, t // BS]) * BS + t % BS for t in range(n)], device=DEV)
+            q = Hy.qk_prep(proj, spec, 0, H * D, (H + G) * D, None, 1e-5, torch.arange(n, device=DEV), kc, vc, slots, dt,
+                           matrix_layout=layout)
+            qs.append(q[starts[s]:])
+        caches[layout] = (torch.cat(qs), kc, vc)
+    q, kc, vc = caches[False]
+    want = Hy.ref_gqa_attention(q.float().cpu(), kc.float().cpu(), vc.float().cpu(), bt, cu, sp, 0.3, None, 0.0, torch.float32,
+                                window, slopes)
+    qm, kcm, vcm = caches[True]
+    got = ops.prefill_attention(qm, kcm, vcm, *gpu(bt, cu, sp), 0.3, window=window, slopes=slopes.to(DEV))
+    torch.testing.assert_close(got.float().cpu().reshape(T, H * D), want, **tol(dt))
+    got = Hy.gqa_attention(qm, kcm, vcm, *gpu(bt, cu, sp), 0.3, None, 0.0, window=window, slopes=slopes.to(DEV),
+                           matrix_layout=True)
+    torch.testing.assert_close(got.float().cpu(), want, **tol(dt))
+    # one row per sequence with split keys on the matrix-core layout
+    B = len(lens)
+    last = torch.tensor([c - 1 for c in ctx], dtype=torch.int32)
+    rows = torch.tensor([int(cu[s + 1]) - 1 for s in range(B)])
+    cu1 = torch.arange(B + 1, dtype=torch.int32)
+    tiles = torch.stack([torch.arange(B), torch.arange(B)], 1).to(torch.int32)
+    got = Hy.gqa_attention(qm[rows.to(DEV)].contiguous(), kcm, vcm, *gpu(bt, cu1, last), 0.3, None, 0.0, tiles=tiles.to(DEV),
+                           num_splits=3, window=window, slopes=slopes.to(DEV), matrix_layout=True)
+    torch.testing.assert_close(got.float().cpu(), want[rows], **tol(dt))
+    # the plain kernels are untouched by the variant: no window, no penalty
+    want0 = Hy.ref_gqa_attention(q.float().cpu(), kc.float().cpu(), vc.float().cpu(), bt, cu, sp, 0.3, None, 0.0, torch.float32)
+    got0 = ops.prefill_attention(qm, kcm, vcm, *gpu(bt, cu, sp), 0.3)
+    torch.testing.assert_close(got0.float().cpu().reshape(T, H * D), want0, **tol(dt))

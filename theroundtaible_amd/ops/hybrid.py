@@ -162,7 +162,8 @@ class SplitWorkspace:
 
 def gqa_attention(q, k_cache, v_cache, block_tables, cu_q, start_pos, scale: float, temp=None, sink: float = 0.0,
                   tiles=None, num_splits: int = 1, workspace: Optional[SplitWorkspace] = None,
-                  out_dtype=None, window: int = 0, slopes=None, gate=None, gate_off: int = 0) -> torch.Tensor:
+                  out_dtype=None, window: int = 0, slopes=None, gate=None, gate_off: int = 0,
+                  matrix_layout: bool = False) -> torch.Tensor:
     """Causal attention of the rows ``q`` [T, H, Dk] (span s = rows ``cu_q[s] .. cu_q[s + 1]`` at
     positions ``start_pos[s] ..`` of sequence s) over the paged keys ``k_cache`` [nb, G, BS, Dk]
     and values ``v_cache`` [nb, G, BS, Dv]: score = q . k * scale (* ``temp[h]``), weights
@@ -170,11 +171,13 @@ def gqa_attention(q, k_cache, v_cache, block_tables, cu_q, start_pos, scale: flo
     device; ``num_splits`` > 1 (one row per span: a decode step) cuts every row's keys into that
     many ranges merged by a second launch. ``window`` > 0: row i sees only keys j with
     i - j < window. ``slopes`` [H] fp32: head h takes slopes[h] * (i - j) off its scores. ``gate``
-    [T, N]: the result is multiplied by sigmoid of its columns ``gate_off .. gate_off + H * Dv``."""
+    [T, N]: the result is multiplied by sigmoid of its columns ``gate_off .. gate_off + H * Dv``.
+    ``matrix_layout`` (GPU): the cache is in the layout of the framework's matrix-core attention
+    kernels (see :func:`qk_prep`), e.g. decode rows of a layer whose prompts run on those kernels."""
     out_dtype = out_dtype or q.dtype
     if _gpu(q):
         T, H, _ = q.shape
-        G, Dv = k_cache.shape[1], v_cache.shape[3]
+        G, Dv = k_cache.shape[1], v_cache.shape[2 if matrix_layout else 3]
         out = torch.empty(T, H * Dv, dtype=out_dtype, device=q.device)
         rows = 1 if num_splits > 1 else rows_per_tile(H // G)
         if tiles is None:
@@ -184,8 +187,11 @@ def gqa_attention(q, k_cache, v_cache, block_tables, cu_q, start_pos, scale: flo
         native().gqa_attention(out, q, k_cache, v_cache, block_tables, cu_q, start_pos, tiles, temp, float(scale),
                                float(sink), rows, int(num_splits),
                                workspace.part_o if num_splits > 1 else None,
-                               workspace.part_ml if num_splits > 1 else None, int(window), slopes, gate, int(gate_off))
+                               workspace.part_ml if num_splits > 1 else None, int(window), slopes, gate, int(gate_off),
+                               1 if matrix_layout else 0)
         return out
+    if matrix_layout:
+        raise ValueError("gqa_attention: the matrix-core cache layout exists on the GPU only")
     return ref_gqa_attention(q, k_cache, v_cache, block_tables, cu_q, start_pos, scale, temp, sink, out_dtype,
                              window, slopes, gate, gate_off)
 
