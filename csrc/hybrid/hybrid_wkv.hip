@@ -42,7 +42,7 @@ __global__ void __launch_bounds__(DB) wkv_scan_kernel(
     const int* __restrict__ cu_q, const int* __restrict__ start_pos, const int* __restrict__ slots,
     const int* __restrict__ chunks, float* __restrict__ ws_e, float* __restrict__ ws_p, int H, int D, float eps) {
   constexpr int SB = stage_rows<DB>();
-  extern __shared__ float lds[];
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   float* sr = lds;                  // [SB][DB] each
   float* sk = sr + SB * DB;
   float* sw = sk + SB * DB;
@@ -116,16 +116,28 @@ __global__ void __launch_bounds__(DB) wkv_scan_kernel(
     }
     __syncthreads();        // the block's r, k, decay are staged
     for (int tt = 0; tt < n; ++tt) {
-      const float* kr = sk + tt * DB;
-      const float* rr = sr + tt * DB;
-      const float* wr = sw + tt * DB;
+      // rows of the block as 16-byte LDS reads (every lane reads the same address: a broadcast)
+      const float4* kr = reinterpret_cast<const float4*>(sk + tt * DB);
+      const float4* rr = reinterpret_cast<const float4*>(sr + tt * DB);
+      const float4* wr = reinterpret_cast<const float4*>(sw + tt * DB);
+      const float4* ur = reinterpret_cast<const float4*>(su);
       const float vj = sv[tt * DB + j];
       float a4[4] = {0.f, 0.f, 0.f, 0.f};     // four partial sums: no 64-long dependent chain
 #pragma unroll
-      for (int i = 0; i < DB; ++i) {
-        const float kv = kr[i] * vj;
-        if (MODE != 1) a4[i & 3] += rr[i] * (S[i] + su[i] * kv);
-        S[i] = wr[i] * S[i] + kv;
+      for (int q = 0; q < DB / 4; ++q) {
+        const float4 k4 = kr[q], w4 = wr[q];
+        const float kv0 = k4.x * vj, kv1 = k4.y * vj, kv2 = k4.z * vj, kv3 = k4.w * vj;
+        if (MODE != 1) {
+          const float4 r4 = rr[q], u4 = ur[q];
+          a4[0] += r4.x * (S[4 * q] + u4.x * kv0);
+          a4[1] += r4.y * (S[4 * q + 1] + u4.y * kv1);
+          a4[2] += r4.z * (S[4 * q + 2] + u4.z * kv2);
+          a4[3] += r4.w * (S[4 * q + 3] + u4.w * kv3);
+        }
+        S[4 * q] = w4.x * S[4 * q] + kv0;
+        S[4 * q + 1] = w4.y * S[4 * q + 1] + kv1;
+        S[4 * q + 2] = w4.z * S[4 * q + 2] + kv2;
+        S[4 * q + 3] = w4.w * S[4 * q + 3] + kv3;
       }
       const float acc = (a4[0] + a4[1]) + (a4[2] + a4[3]);
       if (MODE != 1) {
