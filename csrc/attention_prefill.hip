@@ -41,15 +41,12 @@ struct PrefillCfg {
   static constexpr int VLD = (D * BS * 2) / (256 * 16);
 };
 
-// WIN: the variant with a sliding window (row i sees keys j with 0 <= i - j < window; 0 = none) and a
-// per-head penalty slopes[h] * (i - j) taken off the scaled score; key tiles wholly ahead of the
-// first row's window are not visited.
-template <int D, int HPW, bool WIN = false>
+template <int D, int HPW>
 __global__ void __launch_bounds__(256) prefill_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache,
     const uint16_t* __restrict__ v_cache, const int* __restrict__ block_tables, const int* __restrict__ cu_q,
     const int* __restrict__ start_pos, const int* __restrict__ tile_map, int Hq, int Hkv, int max_blocks,
-    float scale_log2, int rows_per_tile, float sink, int window = 0, const float* __restrict__ slopes = nullptr) {
+    float scale_log2, int rows_per_tile, float sink) {
   using C = PrefillCfg<D>;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
@@ -74,7 +71,6 @@ __global__ void __launch_bounds__(256) prefill_kernel(
   const int tile_rows_end = min(row0 + rows_per_tile, q_end);
   const int kmax = sp + (tile_rows_end - q_begin);  // keys [0, kmax)
   const int ntiles = (kmax + BS - 1) / BS;
-  const int t_first = (WIN && window > 0) ? max(0, sp + (row0 - q_begin) - window + 1) / BS : 0;
 
   // this lane's query row (MFMA column r)
   const int my_row = wrow0 + r;
@@ -91,10 +87,9 @@ __global__ void __launch_bounds__(256) prefill_kernel(
     for (int c = 0; c < D / 32; ++c) qf[hh][c] = *reinterpret_cast<const short8*>(qr + 8 * (4 * c + g));
   }
   float4_ oacc[HPW][D / 16];
-  float m[HPW], lsum[HPW], slope2[HPW];
+  float m[HPW], lsum[HPW];
 #pragma unroll
   for (int hh = 0; hh < HPW; ++hh) {
-    slope2[hh] = (WIN && slopes) ? slopes[min(head0 + hh, hk * G + G - 1)] * LOG2E : 0.f;
     m[hh] = -INFINITY;
     lsum[hh] = 0.f;
 #pragma unroll
@@ -133,13 +128,13 @@ __global__ void __launch_bounds__(256) prefill_kernel(
     }
   };
 
-  if (ntiles > t_first) {
-    gload(t_first);
+  if (ntiles > 0) {
+    gload(0);
     lwrite(0);
   }
   __syncthreads();
-  for (int t = t_first; t < ntiles; ++t) {
-    const int buf = (t - t_first) & 1;
+  for (int t = 0; t < ntiles; ++t) {
+    const int buf = t & 1;
     if (t + 1 < ntiles) gload(t + 1);
     const unsigned char* kb = smem + buf * C::STAGE;
     const unsigned char* vb = kb + C::KBYTES;
@@ -171,12 +166,7 @@ __global__ void __launch_bounds__(256) prefill_kernel(
         for (int i = 0; i < 4; ++i) {
           const int key = key0 + 16 * h + 4 * g + i;
           float v = sc[h][i] * scale_log2;
-          if constexpr (WIN) {
-            const int dist = my_pos - key;
-            v = (dist >= 0 && (window <= 0 || dist < window)) ? v - slope2[hh] * (float)dist : -INFINITY;
-          } else {
-            v = (key <= my_pos) ? v : -INFINITY;
-          }
+          v = (key <= my_pos) ? v : -INFINITY;
           sc[h][i] = v;
           tmax = fmaxf(tmax, v);
         }
@@ -247,7 +237,7 @@ int prefill32_rows(int G);
 int launch_prefill32(void* out, const void* q, const void* k_cache, const void* v_cache, const int* block_tables,
                      const int* cu_q, const int* start_pos, const int* tile_map, int n_tiles, int Hq, int Hkv,
                      int max_blocks, float scale, hipStream_t stream, int map_stride, const int* cmap, int n_split,
-                     float* part_o, float* part_ml, float sink, int window, const float* slopes);
+                     float* part_o, float* part_ml, float sink);
 
 // D = 128 with G <= 8 (a non-power-of-two group in the next power of two of head slots) runs the
 // 32x32-MFMA kernel (attention_prefill32.hip) unless
@@ -266,29 +256,20 @@ int prefill_rows_per_tile(int G, int D) {
 // q [T, Hq, D]; tile_map [n_tiles, 2] int32 (sequence, first row).
 int launch_prefill(void* out, const void* q, const void* k_cache, const void* v_cache, const int* block_tables,
                    const int* cu_q, const int* start_pos, const int* tile_map, int n_tiles, int Hq, int Hkv, int D,
-                   int max_blocks, float scale, hipStream_t stream, float sink, int window, const float* slopes) {
+                   int max_blocks, float scale, hipStream_t stream, float sink) {
   if (n_tiles == 0) return 0;
   const int G = Hq / Hkv;
   if (Hq % Hkv || G < 1 || G > 16) return -1;
   if (use_prefill32(G, D))
     return launch_prefill32(out, q, k_cache, v_cache, block_tables, cu_q, start_pos, tile_map, n_tiles, Hq, Hkv,
-                            max_blocks, scale, stream, 2, nullptr, 0, nullptr, nullptr, sink, window, slopes);
+                            max_blocks, scale, stream, 2, nullptr, 0, nullptr, nullptr, sink);
   const int rows = prefill_rows_per_tile(G, D);
   dim3 grid(n_tiles, Hkv), block(256);
   const float sl2 = scale * LOG2E;
-  const bool win = window > 0 || slopes != nullptr;
 #define RT_PF(DD, HH)                                                                                            \
-  do {                                                                                                           \
-  if (win)                                                                                                       \
-    hipLaunchKernelGGL((prefill_kernel<DD, HH, true>), grid, block, 2 * PrefillCfg<DD>::STAGE, stream,           \
-                       (uint16_t*)out, (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache,   \
-                       block_tables, cu_q, start_pos, tile_map, Hq, Hkv, max_blocks, sl2, rows, sink, window,    \
-                       slopes);                                                                                  \
-  else                                                                                                           \
-    hipLaunchKernelGGL((prefill_kernel<DD, HH, false>), grid, block, 2 * PrefillCfg<DD>::STAGE, stream,          \
-                       (uint16_t*)out, (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache,   \
-                       block_tables, cu_q, start_pos, tile_map, Hq, Hkv, max_blocks, sl2, rows, sink, 0, nullptr); \
-  } while (0)
+  hipLaunchKernelGGL((prefill_kernel<DD, HH>), grid, block, 2 * PrefillCfg<DD>::STAGE, stream, (uint16_t*)out,   \
+                     (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache, block_tables, cu_q, \
+                     start_pos, tile_map, Hq, Hkv, max_blocks, sl2, rows, sink)
   const int hpw = G > 4 ? (G + 3) / 4 : 1;
   if (D == 128) {
     if (hpw == 1) RT_PF(128, 1);
@@ -319,7 +300,7 @@ int launch_prefill_split(void* out, const void* q, const void* k_cache, const vo
   const int G = Hq / Hkv;
   if (Hq % Hkv || !use_prefill32(G, D)) return -1;
   return launch_prefill32(out, q, k_cache, v_cache, block_tables, cu_q, start_pos, items, n_items, Hq, Hkv,
-                          max_blocks, scale, stream, 5, cmap, n_split, part_o, part_ml, 0.f, 0, nullptr);
+                          max_blocks, scale, stream, 5, cmap, n_split, part_o, part_ml, 0.f);
 }
 
 int prefill_split_supported(int G, int D) { return use_prefill32(G, D) ? 1 : 0; }

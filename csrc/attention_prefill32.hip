@@ -105,17 +105,13 @@ struct Loader {
   }
 };
 
-// WIN: the variant with a sliding window (row i sees keys j with 0 <= i - j < window; 0 = none) and a
-// per-head penalty slopes[h] * (i - j) taken off the scaled score: every tile masks per element,
-// the scores are scaled when they are masked, and key tiles ahead of the first row's window are
-// not visited.
-template <int G, int NW, int DEPTH, bool WIN = false>
+template <int G, int NW, int DEPTH>
 __global__ void __launch_bounds__(NW * 64) prefill32_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache,
     const uint16_t* __restrict__ v_cache, const int* __restrict__ block_tables, const int* __restrict__ cu_q,
     const int* __restrict__ start_pos, const int* __restrict__ tile_map, int Hq, int Hkv, int max_blocks,
     float scale_log2, int rows_per_tile, int map_stride, float* __restrict__ part_o, float* __restrict__ part_ml,
-    float sink, int window = 0, const float* __restrict__ slopes = nullptr) {
+    float sink) {
   __shared__ __attribute__((aligned(16))) unsigned char smem[2 * STAGE];   // 68 KiB: static (> 64 KiB)
   // XCD-aware order: workgroups are dealt round-robin over the 8 XCDs (id mod 8), so with
   // id = tile * Hkv + hk every workgroup of kv head hk lands on XCD hk (Hkv = 8): that head's
@@ -147,7 +143,6 @@ __global__ void __launch_bounds__(NW * 64) prefill32_kernel(
     te = min(item[3], te);
     part = item[4];
   }
-  if (WIN && window > 0) tb = max(tb, max(0, sp + (row0 - q_begin) - window + 1) / KT);
   const int ntiles = max(0, te - tb);
   const int my_row = min(wrow0 + c, q_end - 1);
   const int my_pos = sp + (my_row - q_begin);
@@ -155,7 +150,6 @@ __global__ void __launch_bounds__(NW * 64) prefill32_kernel(
   const int wave_rows_end = min(wrow0 + 32, q_end);
   const int wave_kmax = head_ok ? sp + (wave_rows_end - q_begin) : 0;
   const int wave_min_pos = sp + (min(wrow0, q_end - 1) - q_begin);   // first row of the wave
-  const float slope2 = (WIN && slopes) ? slopes[head] * LOG2E : 0.f;
 
   // Q^T B-fragments: lane (q = c, h) holds Q[q][16 dk + 8 h + j]
   short8 qf[D / 16];
@@ -177,7 +171,7 @@ __global__ void __launch_bounds__(NW * 64) prefill32_kernel(
   // one 64-key tile of the math: S^T = K Q^T, online softmax, O^T += V^T P^T
   auto compute_tile = [&](int tl, const unsigned char* kb, const unsigned char* vb) {
       const int t = tb + tl;   // absolute key tile
-      if (tl < ntiles && t * KT < wave_kmax && (!WIN || window <= 0 || (t + 1) * KT > wave_min_pos - window + 1)) {
+      if (tl < ntiles && t * KT < wave_kmax) {
         // ---- S^T = K Q^T (two 32-key blocks) ----
         f16v sc[2];
 #pragma unroll
@@ -198,19 +192,7 @@ __global__ void __launch_bounds__(NW * 64) prefill32_kernel(
         }
         // ---- online softmax down column c: reg i of block blk holds key 64t + 32blk + 16(i>>3) + 8h + (i&7)
         float tmax = -INFINITY;
-        if constexpr (WIN) {                      // window and penalty: per element, scores scaled here
-#pragma unroll
-          for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              const int key = t * KT + 32 * blk + 16 * (i >> 3) + 8 * h + (i & 7);
-              const int dist = my_pos - key;
-              const float v = (dist >= 0 && (window <= 0 || dist < window))
-                                  ? __builtin_fmaf(sc[blk][i], scale_log2, -slope2 * (float)dist) : -INFINITY;
-              sc[blk][i] = v;
-              tmax = fmaxf(tmax, v);
-            }
-        } else if ((t + 1) * KT - 1 <= wave_min_pos) {   // whole tile visible to every row of the wave
+        if ((t + 1) * KT - 1 <= wave_min_pos) {   // whole tile visible to every row of the wave
 #pragma unroll
           for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
@@ -228,7 +210,7 @@ __global__ void __launch_bounds__(NW * 64) prefill32_kernel(
         }
         // scores stay raw: the scale (> 0) commutes with max and is folded into the FMA that
         // feeds exp2 below (one VALU op per score instead of a multiply pass plus a subtract)
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64)) * (WIN ? 1.f : scale_log2);
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64)) * scale_log2;
         // deferred rescale (guide T13): the running max moves only when some column's tile max
         // exceeds it by more than 2^RESCALE (then P <= 2^RESCALE, still exact enough in bf16 and
         // in the f32 sums). Wave-uniform branch, so most tiles skip the 64-multiply O rescale.
@@ -250,9 +232,8 @@ __global__ void __launch_bounds__(NW * 64) prefill32_kernel(
           rt::u32x4 w;
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            const float sf = WIN ? 1.f : scale_log2;    // (WIN: already scaled)
-            const float p0 = rt::fast_exp2(__builtin_fmaf(sc[kc >> 1][8 * (kc & 1) + 2 * j], sf, -msub));
-            const float p1 = rt::fast_exp2(__builtin_fmaf(sc[kc >> 1][8 * (kc & 1) + 2 * j + 1], sf, -msub));
+            const float p0 = rt::fast_exp2(__builtin_fmaf(sc[kc >> 1][8 * (kc & 1) + 2 * j], scale_log2, -msub));
+            const float p1 = rt::fast_exp2(__builtin_fmaf(sc[kc >> 1][8 * (kc & 1) + 2 * j + 1], scale_log2, -msub));
             psum += p0 + p1;
             w[j] = rt::pack2(p0, p1);
           }
@@ -448,15 +429,13 @@ int prefill32_rows(int G) {
 int launch_prefill32(void* out, const void* q, const void* k_cache, const void* v_cache, const int* block_tables,
                      const int* cu_q, const int* start_pos, const int* tile_map, int n_tiles, int Hq, int Hkv,
                      int max_blocks, float scale, hipStream_t stream, int map_stride, const int* cmap, int n_split,
-                     float* part_o, float* part_ml, float sink, int window, const float* slopes) {
+                     float* part_o, float* part_ml, float sink) {
   const int G = Hq / Hkv;
   const int rows = prefill32_rows(G);
   if (rows == 0) return -1;
   if (map_stride != 2 && map_stride != 5) return -2;
   if (map_stride == 5 && n_split > 0 && (cmap == nullptr || part_o == nullptr || part_ml == nullptr)) return -3;
   if (map_stride == 5 && sink != 0.f) return -4;    // the key-split combine has no sink term
-  const bool win = window > 0 || slopes != nullptr;
-  if (map_stride == 5 && win) return -5;            // nor is the key-split plan cut to a window
   const float sl2 = scale * LOG2E;
   dim3 grid(n_tiles * Hkv);
   static const int depth = [] {
@@ -464,11 +443,7 @@ int launch_prefill32(void* out, const void* q, const void* k_cache, const void* 
     return (e && e[0] == '1') ? 1 : 2;
   }();
 #define RT_P32(GG, NWV)                                                                                          \
-  if (win) hipLaunchKernelGGL((prefill32_kernel<GG, NWV, 2, true>), grid, dim3(64 * NWV), 0, stream, (uint16_t*)out,   \
-                     (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache, block_tables, cu_q, \
-                     start_pos, tile_map, Hq, Hkv, max_blocks, sl2, rows, map_stride, part_o, part_ml, sink, window,  \
-                     slopes);                                                                                          \
-  else if (depth == 1) hipLaunchKernelGGL((prefill32_kernel<GG, NWV, 1>), grid, dim3(64 * NWV), 0, stream, (uint16_t*)out, \
+  if (depth == 1) hipLaunchKernelGGL((prefill32_kernel<GG, NWV, 1>), grid, dim3(64 * NWV), 0, stream, (uint16_t*)out, \
                      (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache, block_tables, cu_q, \
                      start_pos, tile_map, Hq, Hkv, max_blocks, sl2, rows, map_stride, part_o, part_ml, sink);          \
   else hipLaunchKernelGGL((prefill32_kernel<GG, NWV, 2>), grid, dim3(64 * NWV), 0, stream, (uint16_t*)out,              \

@@ -30,7 +30,7 @@ int launch_prefill_split(void* out, const void* q, const void* k_cache, const vo
 int prefill_split_supported(int G, int D);
 int launch_prefill(void* out, const void* q, const void* k_cache, const void* v_cache, const int* block_tables,
                    const int* cu_q, const int* start_pos, const int* tile_map, int n_tiles, int Hq, int Hkv, int D,
-                   int max_blocks, float scale, hipStream_t stream, float sink, int window, const float* slopes);
+                   int max_blocks, float scale, hipStream_t stream, float sink);
 int launch_sample(int64_t* out, const void* logits, bool is_bf16, int B, int V, int64_t ld_row,
                   const float* temperature, const float* top_p, const int* top_k, const int64_t* seeds,
                   const int64_t* offsets, float* ws, hipStream_t stream, const void* advance);
@@ -237,18 +237,11 @@ void attn_plan(torch::Tensor plan, int64_t plan_stride, torch::Tensor block_tabl
 
 void prefill_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache, torch::Tensor v_cache,
                        torch::Tensor block_tables, torch::Tensor cu_q, torch::Tensor start_pos, torch::Tensor tile_map,
-                       double scale, double sink, int64_t window, c10::optional<torch::Tensor> slopes) {
+                       double scale, double sink) {
   check_bf16(out, "out");
   check_bf16(q, "q");
   TORCH_CHECK(q.dim() == 3, "q must be [T, Hq, D]");
   const int64_t Hq = q.size(1), D = q.size(2);
-  const float* sl = nullptr;
-  if (slopes.has_value()) {     // per-head distance penalty
-    check_type(*slopes, torch::kFloat32, "slopes");
-    TORCH_CHECK(slopes->numel() == Hq, "slopes must be [Hq]");
-    sl = slopes->data_ptr<float>();
-  }
-  TORCH_CHECK(window >= 0 && window < (int64_t(1) << 31), "window");
   check_caches(k_cache, v_cache, k_cache.size(1), D);
   TORCH_CHECK(k_cache.size(2) == 32, "prefill kernel requires kv block_size == 32");
   check_type(block_tables, torch::kInt32, "block_tables");
@@ -260,7 +253,7 @@ void prefill_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache
   const int rc = launch_prefill(out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                                 block_tables.data_ptr<int>(), cu_q.data_ptr<int>(), start_pos.data_ptr<int>(),
                                 tile_map.data_ptr<int>(), (int)tile_map.size(0), (int)Hq, (int)k_cache.size(1), (int)D,
-                                (int)block_tables.size(1), (float)scale, cur_stream(), (float)sink, (int)window, sl);
+                                (int)block_tables.size(1), (float)scale, cur_stream(), (float)sink);
   TORCH_CHECK(rc == 0, "prefill_attention: unsupported configuration (rc=", rc, ")");
 }
 
@@ -743,7 +736,7 @@ PYBIND11_MODULE(_C, m) {
   m.def("prefill_rows_per_tile", &prefill_rows_per_tile, py::arg("G"), py::arg("D") = 128);
   m.def("prefill_attention", &prefill_attention, py::arg("out"), py::arg("q"), py::arg("k_cache"), py::arg("v_cache"),
         py::arg("block_tables"), py::arg("cu_q"), py::arg("start_pos"), py::arg("tile_map"), py::arg("scale"),
-        py::arg("sink") = 0.0, py::arg("window") = 0, py::arg("slopes") = py::none());
+        py::arg("sink") = 0.0);
   m.def("prefill_attention_split", &prefill_attention_split);
   m.def("prefill_split_supported", &prefill_split_supported, py::arg("G"), py::arg("D") = 128);
   m.def("silu_and_mul", &silu_and_mul);

@@ -604,45 +604,6 @@ def test_decode_steps_on_the_skinny_gemm_and_expert_rows(tmp_path):
     assert float((outs[0] - outs[1]).abs().max()) < 0.25
 
 
-@GPU
-def test_prompts_on_the_matrix_core_attention_kernels(tmp_path, monkeypatch):
-    """Shapes the framework's bf16 matrix-core prompt attention takes (pages of 32, heads of 64 and
-    128): those layers keep their cache in the kernels' layout, prompts and mixed steps run the
-    window / penalty variant, decode rows read the same layout with the any-size kernel. Prompts in
-    portions, a mixed batch and decode steps against the oracle and against the any-size path."""
-    from theroundtaible_amd import ops
-    from theroundtaible_amd.models.retuvik import RetuvikModel
-    if not ops.native_available():
-        pytest.skip("main extension not built")
-    cfg = make_config(width=64, vocab=80, loop=(1, 3, 2),
-                      layers=[att(4, 2, 64, window=40, scale=0.2, mlp={"kind": "dense", "ff": 96}), wkv(2, 32, mlp=None, rank=16),
-                              att(3, 1, 128, window=70, scale=0.15, mlp=moe(4, 2, 32)), att(4, 4, 24, mlp=None)])
-    P = make_checkpoint(tmp_path / "m", cfg, seed=12)
-    ta, tb = toks(150, cfg["vocab"], 12), toks(70, cfg["vocab"], 13)
-    wa, wb = forward(cfg, P, ta), forward(cfg, P, tb)
-    run = ("cuda:0", "bf16")
-    outs = []
-    for matrix in (True, False):
-        monkeypatch.setattr(RetuvikModel, "matrix_attention", matrix)
-        e = engine_for(tmp_path / "m", run, block_size=32, tokens=1024)
-        assert e.kv.matrix == ([True, False, True, False, True, False] if matrix else [False] * 6)
-        ga = [e.step([("a", ta[:100], list(range(100)))])]
-        gb = []
-        o = e.step([("a", ta[100:101], [0]), ("b", tb[:45], list(range(45)))])
-        ga.append(o[:1]), gb.append(o[1:])
-        o = e.step([("a", ta[101:131], list(range(30))), ("b", tb[45:46], [0])])
-        ga.append(o[:30]), gb.append(o[30:])
-        for i in range(19):
-            o = e.step([("a", ta[131 + i:132 + i], [0]), ("b", tb[46 + i:47 + i], [0])])
-            ga.append(o[:1]), gb.append(o[1:])
-        gb.append(e.step([("b", tb[65:], list(range(5)))], end=["a", "b"]))
-        ga, gb = torch.cat(ga), torch.cat(gb)
-        close(ga, wa, run, f"a, matrix={matrix}")
-        close(gb, wb, run, f"b, matrix={matrix}")
-        outs.append((ga, gb))
-    assert float((outs[0][0] - outs[1][0]).abs().max()) < 0.3
-
-
 def test_serving_entry_points_match_run_turns():
     """The continuous-batching entry points (prefill + first token, then decode in chunks while the
     state follows) give the tokens of a single run_turns call; random-init preset weights."""

@@ -55,7 +55,7 @@ def _softplus(v: float) -> float:
 class RetuvikModel(GoganexModel):
     """Shares the row bookkeeping, attention tile maps, split-key workspaces and decode GEMMs of
     :class:`GoganexModel`; the layers, the cache shapes and the forward are its own."""
-    matrix_attention = True        # prompts of layers whose shapes fit run the framework's matrix-core attention kernels
+    matrix_attention = False       # the matrix-core attention kernels know no window or distance penalty
     _DEC_LINEARS = ("w_in", "mix.o", "mix.w1", "mlp.up", "mlp.down")
 
     def __init__(self, cfg: ModelConfig, weights: Dict[str, torch.Tensor], device, dtype=torch.bfloat16,
@@ -115,24 +115,12 @@ class RetuvikModel(GoganexModel):
         return [(m.kv_heads, m.dim, m.vdim) if isinstance(m, GroupedAttentionSpec) else None
                 for m in (ls.mixer for ls in self.cfg.layers)]
 
-    def matrix_layers(self, block_size: int, device, dtype):
-        """Per layer run: whether its prompt attention runs on the framework's bf16 matrix-core
-        kernels (csrc/attention_prefill*.hip, their window / penalty variant): pages of 32 tokens,
-        equal key and value size of 64 or 128, up to 16 query heads per key / value head, the main
-        extension built. Such a run keeps its cache in those kernels' layout; its decode rows read
-        that layout with the any-size kernel. Every other run (and fp32) keeps plain rows."""
-        from .. import ops
-        ok = (self.matrix_attention and torch.device(device).type == "cuda" and dtype == torch.bfloat16
-              and block_size == 32 and ops.native_available())
-        return [bool(ok and isinstance(m, GroupedAttentionSpec) and m.dim == m.vdim and m.dim in (64, 128)
-                     and m.group <= 16 and m.scale > 0) for m in (ls.mixer for ls in self.cfg.layers)]
-
     def make_cache(self, num_blocks: int, block_size: int, device, dtype, n_slots: int):
         from ..engine.kv_cache import GroupedKVCache
         wkv = [isinstance(ls.mixer, WKVSpec) for ls in self.cfg.layers]
         rec = [ls.mixer.state_size if on else 0 for ls, on in zip(self.cfg.layers, wkv)]
         return GroupedKVCache(self.cache_shapes(), self.cfg.hidden, rec, num_blocks, block_size, device, dtype,
-                              n_slots=n_slots, shift_layers=wkv, matrix_layout=self.matrix_layers(block_size, device, dtype))
+                              n_slots=n_slots, shift_layers=wkv)
 
     def cache_bytes_per_block(self, block_size: int, dtype_bytes: int) -> int:
         return max(1, sum(sh[0] * (sh[1] + sh[2]) for sh in self.cache_shapes() if sh is not None)) * block_size * dtype_bytes
@@ -162,28 +150,14 @@ class RetuvikModel(GoganexModel):
         k_off = a.heads * a.dim
         v_off = k_off + a.kv_heads * a.dim
         g_off = v_off + a.kv_heads * a.vdim
-        mx = kv.matrix[l]
         q = Hy.qk_prep(proj, a, 0, k_off, v_off, None, self.cfg.norm_eps, positions, kv.k_layer(l), kv.v_layer(l),
-                       meta.slot_mapping, adt, matrix_layout=mx, q_weight=lw["mix.q.norm"] if a.qk_weight else None,
+                       meta.slot_mapping, adt, q_weight=lw["mix.q.norm"] if a.qk_weight else None,
                        k_weight=lw["mix.k.norm"] if a.qk_weight else None)
-        if mx and not decode:       # prompts (and mixed steps) on the matrix cores; the gate follows
-            from .. import ops
-            rows = ops.native().prefill_rows_per_tile(a.group, a.dim)
-            cache = meta.latent_tiles if meta.latent_tiles is not None else {}
-            meta.latent_tiles = cache
-            tm = cache.get(("matrix", rows))
-            if tm is None:
-                cu, sp = meta.host_rows if meta.host_rows is not None else (b.cu_q.cpu(), b.start_pos.cpu())
-                tm = cache[("matrix", rows)] = ops.prefill_tile_map(cu, rows, sp).to(proj.device, non_blocking=True)
-            o = ops.prefill_attention(q, kv.k_layer(l), kv.v_layer(l), meta.block_tables, b.cu_q, b.start_pos, a.scale, tm,
-                                      sink=a.sink, window=a.window, slopes=lw["slopes"]).reshape(T, a.heads * a.vdim)
-            return o.mul_(torch.sigmoid(proj[:, g_off:g_off + a.heads * a.vdim])) if a.out_gate else o
         splits = self._window_splits(a, T) if decode else 1
         return Hy.gqa_attention(q, kv.k_layer(l), kv.v_layer(l), meta.block_tables, b.cu_q, b.start_pos, a.scale, None,
                                 a.sink, tiles=self._tiles(meta, Hy.rows_per_tile(a.group), b) if proj.is_cuda else None,
                                 num_splits=splits, workspace=self._workspace(T, a, splits), out_dtype=adt,
-                                window=a.window, slopes=lw["slopes"], gate=proj if a.out_gate else None, gate_off=g_off,
-                                matrix_layout=mx)
+                                window=a.window, slopes=lw["slopes"], gate=proj if a.out_gate else None, gate_off=g_off)
 
     def _wkv(self, mix, m, lw, l, src, kv, meta, b, decode, skinny):
         adt = self.dtype

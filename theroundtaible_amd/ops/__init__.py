@@ -313,19 +313,16 @@ def prefill_split_plan(cu_q: torch.Tensor, rows_per_tile: int, start_pos, n_kv_h
 
 def prefill_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                       cu_q: torch.Tensor, start_pos: torch.Tensor, scale: float,
-                      tile_map: Optional[torch.Tensor] = None, split=None, sink: float = 0.0, window: int = 0,
-                      slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      tile_map: Optional[torch.Tensor] = None, split=None, sink: float = 0.0) -> torch.Tensor:
     """``split``: a device-resident :func:`prefill_split_plan` ``(items, cmap, parts)`` — the
     key-split launch + its combine; ``tile_map`` otherwise (whole tiles). ``sink``: a constant
-    added to every softmax denominator as a key of score 0 without a value (whole tiles only).
-    ``window`` > 0: row i sees only keys j with i - j < window; ``slopes`` [Hq] fp32: head h takes
-    slopes[h] * (i - j) off its scaled scores (whole tiles only; a variant of the kernels of its own)."""
+    added to every softmax denominator as a key of score 0 without a value (whole tiles only)."""
     if _use_native(q):
         nat = native()
         out = torch.empty_like(q)
         if split is not None:
-            if sink or window or slopes is not None:
-                raise ValueError("prefill_attention: the key-split launch has no sink, window or penalty")
+            if sink:
+                raise ValueError("prefill_attention: the key-split launch has no sink term")
             items, cmap, parts = split
             hkv, D = k_cache.shape[1], q.shape[2]
             part_o = torch.empty(parts * hkv * 8 * 32 * D, dtype=torch.float32, device=q.device)
@@ -336,11 +333,9 @@ def prefill_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         rows = nat.prefill_rows_per_tile(q.shape[1] // k_cache.shape[1], q.shape[2])
         if tile_map is None:
             tile_map = prefill_tile_map(cu_q.cpu(), rows, start_pos.cpu()).to(q.device)
-        nat.prefill_attention(out, q, k_cache, v_cache, block_tables, cu_q, start_pos, tile_map, scale, float(sink),
-                              int(window), slopes)
+        nat.prefill_attention(out, q, k_cache, v_cache, block_tables, cu_q, start_pos, tile_map, scale, float(sink))
         return out
-    return ref.prefill_attention(q, k_cache, v_cache, block_tables, cu_q.cpu(), start_pos.cpu(), scale, sink=sink,
-                                 window=window, slopes=slopes)
+    return ref.prefill_attention(q, k_cache, v_cache, block_tables, cu_q.cpu(), start_pos.cpu(), scale, sink=sink)
 
 
 PRO_PLAIN, PRO_NORM, PRO_NORM_ADD = 0, 1, 2

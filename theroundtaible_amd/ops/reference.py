@@ -186,10 +186,9 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
 
 def prefill_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       block_tables: torch.Tensor, cu_q: torch.Tensor, start_pos: torch.Tensor,
-                      scale: float, sink: float = 0.0, window: int = 0, slopes=None) -> torch.Tensor:
+                      scale: float, sink: float = 0.0) -> torch.Tensor:
     """Varlen causal attention: sequence s has queries cu_q[s]:cu_q[s+1] at absolute positions
-    start_pos[s] + i, attending to cached keys [0, start_pos[s] + i] — the last ``window`` of them
-    when a window is given; head h takes ``slopes[h] * (i - j)`` off its scaled scores."""
+    start_pos[s] + i, attending to cached keys [0, start_pos[s] + i]."""
     T, Hq, D = q.shape
     Hkv = k_cache.shape[1]
     G = Hq // Hkv
@@ -205,13 +204,8 @@ def prefill_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         sc = torch.einsum("thgd,nhd->thgn", qs, k) * scale
         qpos = torch.arange(st, n)[:, None]
         kpos = torch.arange(n)[None, :]
-        dist = qpos - kpos
-        seen = dist >= 0
-        if window > 0:
-            seen = seen & (dist < window)
-        if slopes is not None:
-            sc = sc - slopes.float().reshape(1, Hkv, G, 1) * dist.float()[:, None, None, :]
-        sc = sc.masked_fill(~seen[:, None, None, :], float("-inf"))
+        mask = (kpos <= qpos)[:, None, None, :]
+        sc = sc.masked_fill(~mask, float("-inf"))
         p = _sink_softmax(sc, sink)
         o = torch.einsum("thgn,nhd->thgd", p, v)
         out[a:b] = o.reshape(b - a, Hq, D).to(q.dtype)
