@@ -118,7 +118,7 @@ def parse():
                         "--compare-layers layers and random weights, through the same engine entry points; "
                         "prints one JSON line per model")
     p.add_argument("--retuvik-large", action="store_true",
-                   help="--arch-compare: run Retuvik presets of width >= 2048 although that run is switched off")
+                   help="--arch-compare: run Retuvik presets at sizes that are switched off (width >= 2048, prompts > 1024)")
     p.add_argument("--compare-layers", type=int, default=4)
     p.add_argument("--compare-prompt", type=int, default=4096, help="--arch-compare: prompt tokens per sequence")
     p.add_argument("--compare-batch", type=int, default=8, help="--arch-compare: sequences decoded together")
@@ -139,11 +139,13 @@ def _arch_compare(args) -> int:
     for pair in filter(None, args.arch_compare.split(",")):
         for name in pair.split(":"):
             base = get_config(name)
-            if base.arch == "retuvik" and base.hidden >= 2048 and device != "cpu" and not args.retuvik_large:
-                # the one run at these sizes (retuvik-8b, 4 layers, 4096-token prompts) ended in a GPU memory
-                # fault whose cause has not been found; the path stays off until it is
-                raise SystemExit(f"--arch-compare {name}: switched off at this size (the one run so far ended in a GPU "
-                                 f"memory fault whose cause is not found); --retuvik-large runs it regardless")
+            if (base.arch == "retuvik" and (base.hidden >= 2048 or P > 1024) and device != "cpu"
+                    and not args.retuvik_large):
+                # two runs at such sizes (retuvik-8b; retuvik-0.5b with 4096-token prompts, beside other
+                # programs in one call) ended in GPU memory faults whose cause has not been found
+                raise SystemExit(f"--arch-compare {name}: switched off above width 2047 or --compare-prompt 1024 (runs "
+                                 f"at such sizes ended in a GPU memory fault whose cause is not found); "
+                                 f"--retuvik-large runs it regardless")
             ov = {"n_layers": L}
             if base.layers is not None:
                 ov["layers"] = tuple(base.layers[:L])
