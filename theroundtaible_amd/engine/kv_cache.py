@@ -306,11 +306,16 @@ class GroupedKVCache(StatefulPagedCache):
     States, fp32, one row per slot: ``shift[l]`` ``[n_slots, width]`` is the previous token's
     normed mixer input (token shift; None for a run without one when ``shift_layers`` says so);
     ``rec[l]`` ``[n_slots, rec_width_l]`` the state of the layer's recurrence — a channel vector,
-    or the flattened heads x dim x dim matrix state of a wkv mixer (None for a layer without one).
+    or the flattened matrix state per head of a wkv / delta-rule mixer (None for a layer without
+    one). ``canon_taps`` > 1: ``conv[l]`` ``[n_slots, 2, canon_taps - 1, width]`` holds the last
+    inputs of the layer's two input convolutions (mixer, feed-forward), oldest first.
+    ``short_conv[l]`` = (channels, taps): ``sconv[l]`` ``[n_slots, taps - 1, channels]`` holds the
+    last inputs of a short convolution inside the mixer (None for a layer without one).
     A sequence at position 0 never reads its slot, so a reused slot needs no clearing."""
 
     def __init__(self, shapes, width: int, rec_widths, num_blocks: int, block_size: int, device,
-                 dtype=torch.bfloat16, n_slots: int = 16, matrix_layout=None, shift_layers=None):
+                 dtype=torch.bfloat16, n_slots: int = 16, matrix_layout=None, shift_layers=None,
+                 canon_taps: int = 0, short_conv=None):
         shapes = [sh if sh is not None else (0, 0, 0) for sh in shapes]
         self.n_layers = len(shapes)
         # per run: the layout of the framework's matrix-core attention kernels (keys chunk-major
@@ -333,10 +338,16 @@ class GroupedKVCache(StatefulPagedCache):
         self.shift = [torch.zeros(n_slots, width, dtype=torch.float32, device=device) if on else None
                       for on in shift_layers]
         self.rec = [torch.zeros(n_slots, w, dtype=torch.float32, device=device) if w else None for w in rec_widths]
+        self.canon_taps = canon_taps
+        self.conv = [torch.zeros(n_slots, 2, max(canon_taps - 1, 1), width, dtype=torch.float32, device=device)
+                     if canon_taps > 0 else None for _ in self.shapes]
+        short_conv = list(short_conv) if short_conv is not None else [None] * len(self.shapes)
+        self.sconv = [torch.zeros(n_slots, max(sc[1] - 1, 1), sc[0], dtype=torch.float32, device=device)
+                      if sc is not None else None for sc in short_conv]
 
     @staticmethod
     def bytes_per_block(shapes, block_size, dtype_bytes=2) -> int:   # type: ignore[override]
-        return sum(g * (dk + dv) for g, dk, dv in shapes) * block_size * dtype_bytes
+        return sum(g * (dk + dv) for g, dk, dv in shapes if g) * block_size * dtype_bytes
 
     def k_layer(self, l: int) -> torch.Tensor:
         return self.k[l]
@@ -352,4 +363,4 @@ class GroupedKVCache(StatefulPagedCache):
                 t.index_copy_(0, di, t.index_select(0, si))
 
     def state_tensors(self) -> List[torch.Tensor]:
-        return [t for t in self.shift + self.rec if t is not None]
+        return [t for t in self.shift + self.rec + self.conv + self.sconv if t is not None]

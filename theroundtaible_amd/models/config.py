@@ -2,6 +2,7 @@
 from __future__ import annotations
 
 import json
+import math
 import os
 from dataclasses import dataclass, replace
 from typing import Callable, Dict, Optional, Tuple
@@ -35,6 +36,7 @@ class RotarySpec:
     base: float
     dims: int
     scaling: Optional[tuple] = None
+    halves: bool = False      # entry i pairs with i + dims / 2 instead of 2i with 2i + 1
 
 
 @dataclass(frozen=True)
@@ -52,7 +54,14 @@ class GroupedAttentionSpec:
     ``q.norm`` / ``k.norm``, shared by the heads). ``q_temp`` = (coef, every): the queries of
     position p are multiplied by 1 + coef * ln(floor((p + 1) / every) + 1). ``value_norm``: every
     value head is divided by its root mean square before it is cached. ``out_gate``: the
-    concatenated heads are multiplied by sigmoid(W_g h) ahead of the output projection."""
+    concatenated heads are multiplied by sigmoid(W_g h) ahead of the output projection.
+    ``softcap`` > 0: scores become softcap * tanh(score / softcap). ``wide_norm``: instead of the
+    per-head unit RMS, the whole query projection (and the whole key projection) is divided by
+    its root mean square over all heads at once and multiplied by a weight per channel (tensors
+    ``q.norm`` / ``k.norm`` of the projection's size), BEFORE the rotation. ``bias``: the query and
+    key projections add a bias (tensors ``q.b`` / ``k.b``). ``value_rot``: the value of position j
+    is turned by j over all its entries before it is cached (pair m by j * base^(-2m / vdim), the
+    pairs laid out as the key rotation's), and each head's output at position i is turned back by i."""
     heads: int
     kv_heads: int
     dim: int
@@ -68,6 +77,10 @@ class GroupedAttentionSpec:
     q_temp: Optional[Tuple[float, int]] = None
     value_norm: bool = False
     out_gate: bool = False
+    softcap: float = 0.0
+    wide_norm: bool = False
+    bias: bool = False
+    value_rot: Optional[RotarySpec] = None
 
     @property
     def group(self) -> int:
@@ -87,11 +100,72 @@ class MinGRUSpec:
 
 
 @dataclass(frozen=True)
+class DecaySumSpec:
+    """Linear attention with one constant decay per head (lightning attention): per head a
+    ``dim`` x ``vdim`` fp32 state, S_t = decay S_(t-1) + k_t v_t^T, o_t = S_t^T q_t, with
+    q, k, v = silu of their projections; the concatenated heads are RMS-normed together, weighted,
+    and gated by sigmoid of a fourth projection."""
+    heads: int
+    dim: int
+    vdim: int
+    decay: Tuple[float, ...]
+
+    @property
+    def state_size(self) -> int:
+        return self.heads * self.dim * self.vdim
+
+
+@dataclass(frozen=True)
+class RemovalSpec:
+    """Generalized delta rule: per head a ``dim`` x ``dim`` fp32 state with a per-token,
+    per-channel decay w (a low-rank path through tanh, then exp(-e^(-1/2) sigmoid(.))) and a
+    per-channel removal rate a = sigmoid(W_a h + b): with u the unit-length key,
+    S_t = diag(w_t) S_(t-1) - (a_t * u_t)(u_t^T S_(t-1)) + k_t v_t^T, o_t = S_t^T r_t; each head
+    is divided by its root mean square, weighted, and gated by sigmoid of a projection."""
+    heads: int
+    dim: int
+    decay_rank: int = 0
+
+    @property
+    def vdim(self) -> int:
+        return self.dim
+
+    @property
+    def state_size(self) -> int:
+        return self.heads * self.dim * self.dim
+
+
+@dataclass(frozen=True)
+class DeltaSpec:
+    """Gated delta rule: ``heads`` value heads of size ``vdim`` over ``kv_heads`` query / key heads
+    of size ``dim``; q, k, v pass a causal convolution of ``conv`` taps per channel and silu, q and
+    k are made unit vectors (q also times dim^(-1/2)); one decay g and one step size beta per head
+    and token: S <- g S; S <- S + k (beta (v - S^T k))^T; o = S^T q. Each head is divided by its
+    root mean square, weighted (one weight vector shared by the heads), gated by silu of a projection."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int
+
+    @property
+    def state_size(self) -> int:
+        return self.heads * self.dim * self.vdim
+
+    @property
+    def conv_channels(self) -> int:
+        return 2 * self.kv_heads * self.dim + self.heads * self.vdim
+
+
+@dataclass(frozen=True)
 class ParallelSpec:
-    """Two mixers reading the same input: attention (``left``) and a minGRU (``right``); the layer
-    adds half the sum of their RMS-normed outputs."""
+    """Two mixers reading the same input: attention (``left``) beside a recurrence (``right``: a
+    minGRU, whose layer adds half the sum of the two RMS-normed outputs; or a matrix-state
+    recurrence, whose layer adds ``left_scale`` * left + ``right_scale`` * right)."""
     left: GroupedAttentionSpec
-    right: MinGRUSpec
+    right: object
+    left_scale: float = 0.5
+    right_scale: float = 0.5
 
 
 @dataclass(frozen=True)
@@ -115,11 +189,16 @@ class WKVSpec:
 
 @dataclass(frozen=True)
 class MoESpec:
-    """Mixture of gated feed-forward experts: ``experts`` experts of width ``ff``, each token runs
-    the ``top`` with the largest router logits, weighted by the softmax over those logits alone."""
+    """Mixture of feed-forward experts: ``experts`` experts of width ``ff``, each token runs the
+    ``top`` with the largest router logits, weighted by the softmax over those logits alone (which
+    equals the softmax over all experts renormalised over the chosen ones). ``act`` "silu_glu":
+    W_down (silu(W_gate h) * W_up h); "relu2": W_down relu(W_up h)^2. ``shared_ff`` > 0: one more
+    expert of that width (tensors ``shared.*``) runs for every token with weight 1."""
     experts: int
     top: int
     ff: int
+    act: str = "silu_glu"
+    shared_ff: int = 0
 
 
 @dataclass(frozen=True)
@@ -182,7 +261,7 @@ class ModelConfig:
 
     def n_params(self) -> int:
         h, f, v, L = self.hidden, self.ffn, self.vocab, self.n_layers
-        if self.arch in ("goganex", "retuvik"):
+        if self.arch in ("goganex", "retuvik", "ledinex"):
             from .weights import layout_for
             n = 0
             for shape, _, _ in layout_for(self).values():
@@ -290,7 +369,7 @@ def parse_mupulorn(d: dict, name: str = "mupulorn") -> ModelConfig:
 def attention_of(ls: LayerSpec):
     """The attention part of a layer's mixer (the left half of a parallel mixer; None for a
     mixer without attention)."""
-    if isinstance(ls.mixer, WKVSpec):
+    if isinstance(ls.mixer, (WKVSpec, DeltaSpec)):
         return None
     return ls.mixer.left if isinstance(ls.mixer, ParallelSpec) else ls.mixer
 
@@ -459,6 +538,117 @@ def retuvik_config(name: str, n_layers: int, width: int, heads: int, kv_heads: i
     return parse_retuvik(d, name)
 
 
+def _ledinex_attention(mx: dict, kind: str, where: str) -> GroupedAttentionSpec:
+    r = mx["rot"]
+    sc = r.get("scaling")
+    scaling = None
+    if sc is not None and "original" in sc:       # blended frequencies and enlarged cos / sin (YaRN)
+        f = float(sc["factor"])
+        scaling = ("yarn", f, float(sc["original"]), float(sc["fast"]), float(sc["slow"]), 0.1 * math.log(f) + 1.0)
+    elif sc is not None:
+        scaling = ("linear", float(sc["factor"]))
+    rot = RotarySpec(float(r["base"]), int(r["dims"]), scaling, halves=True)
+    two = kind == "parallel_2"
+    mask = mx.get("mask")
+    vdim = int(mx["vdim"])
+    a = GroupedAttentionSpec(int(mx["heads"]), int(mx["kv_heads"]), int(mx["dim"]), vdim, float(mx["scale"]), rot,
+                             value_from_key=two, window=int(mask["size"]) if mask is not None else 0,
+                             softcap=float(mx.get("softcap") or 0.0), wide_norm=True, bias=two,
+                             value_rot=None if two else RotarySpec(rot.base, vdim, None, halves=True))
+    if a.heads % a.kv_heads:
+        raise ValueError(f"{where}: {a.heads} query heads do not divide over {a.kv_heads} key/value heads")
+    if rot.dims > a.dim or rot.dims % 2 or (a.value_rot is not None and vdim % 2):
+        raise ValueError(f"{where}: rot.dims {rot.dims} / vdim {vdim} do not fit the rotation")
+    if a.value_from_key and a.vdim != a.dim:
+        raise ValueError(f"{where}: values are the keys, so vdim {a.vdim} must equal dim {a.dim}")
+    if a.window < 0:
+        raise ValueError(f"{where}: mask.size out of range")
+    return a
+
+
+def parse_ledinex(d: dict, name: str = "ledinex") -> ModelConfig:
+    """``config.json`` of a Ledinex checkpoint -> :class:`ModelConfig`. Every layer is a mixer of
+    type "parallel" (attention with turned values and soft-capped scores beside a constant-decay
+    linear attention), "parallel_2" (windowed attention whose values are its keys beside a
+    generalized delta rule) or "delta" (a gated delta rule), and a mixture of squared-ReLU experts
+    with a shared expert (or no feed-forward). A key the file does not have switches its mechanism
+    off (no window, no soft cap, no frequency scaling, no shared expert)."""
+    specs = []
+    for i, e in enumerate(d["layers"]):
+        where, kind, mx = f"{name}: layer {i}", e["type"], e["mixer"]
+        if kind == "delta":
+            mixer = DeltaSpec(int(mx["heads"]), int(mx["kv_heads"]), int(mx["dim"]), int(mx["vdim"]), int(mx["conv"]))
+            if mixer.heads % mixer.kv_heads or mixer.conv < 1:
+                raise ValueError(f"{where}: heads {mixer.heads} / kv_heads {mixer.kv_heads} / conv {mixer.conv}")
+        elif kind in ("parallel", "parallel_2"):
+            left, rx = _ledinex_attention(mx["left"], kind, where), mx["right"]
+            if kind == "parallel":
+                right = DecaySumSpec(int(rx["heads"]), int(rx["dim"]), int(rx.get("vdim", rx["dim"])),
+                                     tuple(float(v) for v in rx["decay"]))
+                if len(right.decay) != right.heads:
+                    raise ValueError(f"{where}: {len(right.decay)} decays for {right.heads} heads")
+            else:
+                right = RemovalSpec(int(rx["heads"]), int(rx["dim"]), int(rx.get("decay_rank", 0)))
+            mixer = ParallelSpec(left, right, float(mx["left_scale"]), float(mx["right_scale"]))
+        else:
+            raise ValueError(f"{where}: unknown mixer type '{kind}'")
+        mlp = e.get("mlp")
+        if mlp is None:
+            specs.append(LayerSpec(kind, mixer, 0, "moe", i))
+        elif mlp.get("kind") == "moe":
+            sh = mlp.get("shared")
+            moe = MoESpec(int(mlp["router"]["experts"]), int(mlp["router"]["top"]), int(mlp["expert"]["ff"]), "relu2",
+                          int(sh["ff"]) if sh is not None else 0)
+            if not 1 <= moe.top <= moe.experts:
+                raise ValueError(f"{where}: top {moe.top} of {moe.experts} experts")
+            specs.append(LayerSpec(kind, mixer, moe.ff, "moe", i, moe=moe))
+        else:
+            raise ValueError(f"{where}: unknown feed-forward kind '{mlp.get('kind')}'")
+    atts = [attention_of(s) for s in specs if attention_of(s) is not None]
+    top = max(atts, key=lambda m: m.heads) if atts else None
+    any_mixer = specs[0].mixer
+    taps = int(d["canon"]["taps"])
+    if not 1 <= taps <= 16:
+        raise ValueError(f"{name}: canon.taps {taps} out of range")
+    return ModelConfig(name, "ledinex", len(specs), int(d["width"]), top.heads if top else any_mixer.heads,
+                       top.kv_heads if top else any_mixer.kv_heads, top.dim if top else any_mixer.dim,
+                       max([s.ff for s in specs] + [0]), int(d["vocab"]), int(d.get("max_pos", 1 << 17)), 0.0,
+                       float(d["norm"]["eps"]), tie_embeddings=True, layers=tuple(specs), canon_taps=taps,
+                       logit_scale=float(d.get("logit_scale", 1.0)),
+                       embed_scale=float(d.get("embedding", {}).get("scale", 1.0)))
+
+
+def ledinex_config(name: str, n_layers: int, width: int, heads: int, kv_heads: int, dim: int, ff: int, vocab: int,
+                   pattern: Tuple[str, ...] = ("parallel_2", "delta", "parallel"), rec_heads: int = 0, rec_dim: int = 64,
+                   window: int = 1024, experts: int = 8, top: int = 2, expert_ff: int = 0, shared_ff: int = 0,
+                   taps: int = 3, conv: int = 4, decay_rank: int = 64, max_pos: int = 1 << 17) -> ModelConfig:
+    """A Ledinex stack from a few sizes (benchmarks and presets): the mixer types of ``pattern``
+    in turn; every feed-forward a mixture of ``experts`` squared-ReLU experts (``top`` per token,
+    together ``ff`` wide unless ``expert_ff`` is given) plus a shared expert."""
+    A = rec_heads or width // rec_dim
+    eff = expert_ff or max(32, ff // (top + 1))
+    mlp = {"kind": "moe", "expert": {"ff": eff}, "router": {"experts": experts, "top": top},
+           "shared": {"ff": shared_ff or eff}} if ff else None
+    left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5}
+    kinds = {
+        "parallel": {"left": dict(left, softcap=30.0, rot={"base": 500000.0, "dims": dim, "scaling": {"factor": 4.0}}),
+                     "left_scale": 0.7, "right_scale": 0.7,
+                     "right": {"heads": A, "dim": rec_dim, "vdim": rec_dim,
+                               "decay": [math.exp(-2.0 ** (-1 - 5.0 * a / max(1, A - 1))) for a in range(A)]}},
+        "parallel_2": {"left": dict(left, mask={"size": window},
+                                    rot={"base": 50000.0, "dims": dim // 2,
+                                         "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}),
+                       "left_scale": 0.7, "right_scale": 0.7,
+                       "right": {"heads": A, "dim": rec_dim, "decay_rank": decay_rank}},
+        "delta": {"heads": A, "kv_heads": max(1, A // 2), "dim": rec_dim, "vdim": rec_dim, "conv": conv},
+    }
+    layers = [{"type": pattern[i % len(pattern)], "mixer": kinds[pattern[i % len(pattern)]], "mlp": mlp}
+              for i in range(n_layers)]
+    return parse_ledinex({"architecture": "Ledinex", "canon": {"taps": taps}, "embedding": {"scale": 1.0},
+                          "layers": layers, "logit_scale": 1.0, "norm": {"eps": 1e-5}, "vocab": vocab, "width": width,
+                          "max_pos": max_pos}, name)
+
+
 def mupulorn_config(name: str, n_layers: int, width: int, heads: int, dim: int, rot_dim: int, vdim: int,
                     kv_rank: int, q_rank: int, ff: int, vocab: int, taps: int = 4, shared_every: int = 0,
                     rot_base: float = 10000.0, max_pos: int = 1 << 17) -> ModelConfig:
@@ -482,7 +672,7 @@ def mupulorn_config(name: str, n_layers: int, width: int, heads: int, dim: int, 
 
 # config.json "architecture" -> parser (checkpoint directories name their own model class)
 ARCHITECTURES: Dict[str, Callable[[dict, str], ModelConfig]] = {"Mupulorn": parse_mupulorn, "Goganex": parse_goganex,
-                                                                "Retuvik": parse_retuvik}
+                                                                "Retuvik": parse_retuvik, "Ledinex": parse_ledinex}
 
 PRESETS.update({
     # Mupulorn (latent attention + input convolutions + PolyNorm feed-forward), random-init sizes:
@@ -520,6 +710,17 @@ PRESETS.update({
     "retuvik-1b": retuvik_config("retuvik-1b", 16, 2048, 32, 8, 64, 8192, 128256, moe_every=4),
     "retuvik-3b": retuvik_config("retuvik-3b", 28, 3072, 24, 8, 128, 8192, 128256, moe_every=4),
     "retuvik-8b": retuvik_config("retuvik-8b", 32, 4096, 32, 8, 128, 14336, 128256, moe_every=4),
+})
+
+PRESETS.update({
+    # Ledinex (input convolutions, post-norm sublayers, attention beside a matrix-state recurrence,
+    # gated delta rule layers, squared-ReLU experts with a shared expert), random-init sizes: a
+    # test-sized stack and stacks whose layers have the shapes of 0.5B (Qwen2.5) / 1B / 3B-class models
+    "tiny-ledinex": ledinex_config("tiny-ledinex", 3, 128, 4, 2, 32, 192, 32000, rec_heads=2, rec_dim=32, window=24,
+                                   experts=6, top=2, expert_ff=48, shared_ff=80, decay_rank=8),
+    "ledinex-0.5b": ledinex_config("ledinex-0.5b", 24, 896, 14, 2, 64, 4864, 151936),      # Qwen2.5-0.5B's sizes
+    "ledinex-1b": ledinex_config("ledinex-1b", 16, 2048, 32, 8, 64, 8192, 128256),
+    "ledinex-3b": ledinex_config("ledinex-3b", 28, 3072, 24, 8, 128, 8192, 128256, rec_dim=128),
 })
 
 

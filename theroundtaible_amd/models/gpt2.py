@@ -95,5 +95,8 @@ def build_model(cfg: ModelConfig, weights, device, dtype=torch.bfloat16, tp: Opt
     if cfg.arch == "retuvik":
         from .retuvik import RetuvikModel
         return RetuvikModel(cfg, weights, device, dtype, tp)
+    if cfg.arch == "ledinex":
+        from .ledinex import LedinexModel
+        return LedinexModel(cfg, weights, device, dtype, tp)
     from .llama import LlamaModel
     return LlamaModel(cfg, weights, device, dtype, tp)

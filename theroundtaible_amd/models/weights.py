@@ -211,6 +211,77 @@ def retuvik_layout(cfg: ModelConfig) -> Dict[str, Tuple[Tuple[int, ...], str, Op
     return lay
 
 
+def ledinex_layout(cfg: ModelConfig) -> Dict[str, Tuple[Tuple[int, ...], str, Optional[str]]]:
+    """Checkpoint names and shapes of a Ledinex model (linear weights [out, in]). The logits read
+    the embedding table, so there is no head tensor. The rank of a generalized-delta mixer's decay
+    path is whatever ``w1`` / ``w2`` have (-1 in the shape) unless the spec names one. Not
+    tensor-parallel: every kind is None."""
+    from .config import DecaySumSpec, DeltaSpec, RemovalSpec
+    W = cfg.hidden
+    lay: Dict[str, Tuple[Tuple[int, ...], str, Optional[str]]] = {
+        "embed": ((cfg.vocab, W), "normal", None),
+        "final.norm": ((W,), "zeros", None),
+    }
+    for i, ls in enumerate(cfg.layers):
+        p, m = f"l{i}.", ls.mixer
+        lay[p + "norm1"] = ((W,), "zeros", None)
+        lay[p + "canon1"] = ((W, cfg.canon_taps), "small", None)
+        if isinstance(m, DeltaSpec):
+            q = p + "mix."
+            for n, rows in (("q", m.kv_heads * m.dim), ("k", m.kv_heads * m.dim), ("v", m.heads * m.vdim)):
+                lay[q + n] = ((rows, W), "normal", None)
+                lay[q + n + ".conv"] = ((rows, m.conv), "conv", None)
+            lay[q + "b"] = ((m.heads, W), "normal", None)
+            lay[q + "a"] = ((m.heads, W), "normal", None)
+            lay[q + "A_log"] = ((m.heads,), "zeros", None)
+            lay[q + "dt_bias"] = ((m.heads,), "zeros", None)
+            lay[q + "norm"] = ((m.vdim,), "ones", None)
+            lay[q + "g"] = ((m.heads * m.vdim, W), "normal", None)
+            lay[q + "o"] = ((W, m.heads * m.vdim), "normal", None)
+        else:
+            a, r = m.left, m.right
+            q = p + "mix.left."
+            lay[q + "q"] = ((a.heads * a.dim, W), "normal", None)
+            lay[q + "k"] = ((a.kv_heads * a.dim, W), "normal", None)
+            if a.bias:
+                lay[q + "q.b"] = ((a.heads * a.dim,), "zeros", None)
+                lay[q + "k.b"] = ((a.kv_heads * a.dim,), "zeros", None)
+            if not a.value_from_key:
+                lay[q + "v"] = ((a.kv_heads * a.vdim, W), "normal", None)
+            lay[q + "q.norm"] = ((a.heads * a.dim,), "ones", None)
+            lay[q + "k.norm"] = ((a.kv_heads * a.dim,), "ones", None)
+            lay[q + "o"] = ((W, a.heads * a.vdim), "normal", None)
+            q = p + "mix.right."
+            if isinstance(r, DecaySumSpec):
+                lay[q + "q"] = ((r.heads * r.dim, W), "normal", None)
+                lay[q + "k"] = ((r.heads * r.dim, W), "normal", None)
+                lay[q + "v"] = ((r.heads * r.vdim, W), "normal", None)
+            elif isinstance(r, RemovalSpec):
+                rank = r.decay_rank or -1
+                for n in "rkv":
+                    lay[q + n] = ((r.heads * r.dim, W), "normal", None)
+                lay[q + "a"] = ((r.heads * r.dim, W), "normal", None)
+                lay[q + "a.b"] = ((r.heads * r.dim,), "zeros", None)
+                lay[q + "w1"] = ((rank, W), "normal", None)
+                lay[q + "w2"] = ((r.heads * r.dim, rank), "normal", None)
+                lay[q + "w0"] = ((r.heads * r.dim,), "zeros", None)
+            lay[q + "g"] = ((r.heads * r.vdim, W), "normal", None)
+            lay[q + "norm"] = ((r.heads * r.vdim,), "ones", None)
+            lay[q + "o"] = ((W, r.heads * r.vdim), "normal", None)
+        if not ls.ff:
+            continue
+        lay[p + "norm2"] = ((W,), "zeros", None)
+        lay[p + "canon2"] = ((W, cfg.canon_taps), "small", None)
+        for e in range(ls.moe.experts):
+            lay[p + f"mlp.e{e}.up"] = ((ls.ff, W), "normal", None)
+            lay[p + f"mlp.e{e}.down"] = ((W, ls.ff), "normal", None)
+        lay[p + "mlp.router"] = ((ls.moe.experts, W), "normal", None)
+        if ls.moe.shared_ff:
+            lay[p + "mlp.shared.up"] = ((ls.moe.shared_ff, W), "normal", None)
+            lay[p + "mlp.shared.down"] = ((W, ls.moe.shared_ff), "normal", None)
+    return lay
+
+
 def layout_for(cfg: ModelConfig):
     if cfg.arch == "mupulorn":
         return mupulorn_layout(cfg)
@@ -218,6 +289,8 @@ def layout_for(cfg: ModelConfig):
         return goganex_layout(cfg)
     if cfg.arch == "retuvik":
         return retuvik_layout(cfg)
+    if cfg.arch == "ledinex":
+        return ledinex_layout(cfg)
     return gpt2_layout(cfg) if cfg.arch == "gpt2" else llama_layout(cfg)
 
 
@@ -302,6 +375,11 @@ def _init(shape, init, std, g, device, dtype):
         return torch.full(shape, 0.5, device=device, dtype=dtype)
     if init == "poly":      # PolyNorm coefficients: equal thirds, no offset
         return torch.tensor([1 / 3, 1 / 3, 1 / 3, 0.0], device=device, dtype=dtype)
+    if init == "conv":      # short convolution ahead of an activation: most of the weight on the current token
+        w = torch.empty(shape, device=device, dtype=dtype)
+        w.normal_(0.0, 0.1, generator=g)
+        w[..., -1] += 1.0
+        return w
     if init == "small":     # input-convolution taps
         w = torch.empty(shape, device=device, dtype=dtype)
         w.normal_(0.0, 0.1, generator=g)
@@ -372,7 +450,7 @@ def load_safetensors(cfg: ModelConfig, path: str, device, dtype, tp: TPInfo) -> 
         tensors.update(load_file(f, device="cpu"))
     lay = layout_for(cfg)
     out = {}
-    if cfg.arch in ("mupulorn", "goganex", "retuvik"):
+    if cfg.arch in ("mupulorn", "goganex", "retuvik", "ledinex"):
         # the checkpoint's own names; integer tables keep their type, everything else takes `dtype`
         if tp.size > 1:
             raise ValueError(f"{cfg.arch} checkpoints are not tensor-parallel")

@@ -51,7 +51,7 @@ def main(argv=None) -> int:
         if arch == "mupulorn":
             from .ops import latent
             latent.ensure_built()
-        elif arch in ("goganex", "retuvik"):
+        elif arch in ("goganex", "retuvik", "ledinex"):
             from .ops import hybrid
             hybrid.ensure_built()
     bs = a.block_size
