@@ -7,6 +7,8 @@
 //                 and i - j < window when a window is given (tiles wholly ahead of it are skipped)
 //   weight_j   = exp(s_j) / (sink + sum_j exp(s_j))        (sink: a key of score 0 without a value)
 //   out       *= sigmoid(gate[row, h * Dv + col])          when a gate is given
+//   with a soft cap c the scaled score becomes c * tanh(score / c) ahead of the distance term; the
+//   result is multiplied by out_scale and may land in a column range of a wider buffer
 //
 // One workgroup of 4 waves = one work item (sequence, first row) x one key/value head x one key
 // range: up to 32 (row, head) pairs, 8 per wave, that all read the same keys and values. The keys
@@ -37,7 +39,7 @@ __global__ void __launch_bounds__(256) gqa_attention_kernel(
     const int* __restrict__ tiles, const float* __restrict__ temp, float* __restrict__ part_o,
     float* __restrict__ part_ml, int H, int G, int Dk, int Dv, int BS, int max_blocks, int R, int KT, int hchunks,
     float scale, float sink, int window, const float* __restrict__ slopes, const T* __restrict__ gate,
-    int gate_stride, int layout) {
+    int gate_stride, int layout, float softcap, float out_scale, int out_stride, int out_off) {
   extern __shared__ float lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int seq = tiles[2 * blockIdx.x], row0 = tiles[2 * blockIdx.x + 1];
@@ -121,7 +123,9 @@ __global__ void __launch_bounds__(256) gqa_attention_kernel(
     for (int i = 0; i < kPW; ++i) {
       const int dist = qpos[i] - (kb + lane);
       const bool ok = lane < KT && dist >= 0 && (window <= 0 || dist < window);
-      const float sc = ok ? s[i] * hs[i] - sl[i] * (float)dist : kNeg;
+      float raw = s[i] * hs[i];
+      if (softcap > 0.f) raw = softcap * tanhf(raw / softcap);
+      const float sc = ok ? raw - sl[i] * (float)dist : kNeg;
       const float mn = fmaxf(m[i], rt::wave_max(sc));
       const float pe = ok ? __expf(sc - mn) : 0.f;
       alpha[i] = __expf(m[i] - mn);
@@ -162,9 +166,9 @@ __global__ void __launch_bounds__(256) gqa_attention_kernel(
       for (int c = 0; c < DVL; ++c) {
         const int col = lane + 64 * c;
         if (col < Dv) {
-          float v = o[i][c] * inv;
+          float v = o[i][c] * inv * out_scale;
           if (gate) v *= 1.0f / (1.0f + __expf(-DT<T>::load(gate + (size_t)(row0 + r) * gate_stride + h * Dv + col)));
-          DT<T>::store(out + rh * Dv + col, v);
+          DT<T>::store(out + (size_t)(row0 + r) * out_stride + out_off + h * Dv + col, v);
         }
       }
     } else {
@@ -186,7 +190,8 @@ __global__ void __launch_bounds__(256) gqa_attention_kernel(
 template <typename T>
 __global__ void __launch_bounds__(64) gqa_combine_kernel(T* __restrict__ out, const float* __restrict__ part_o,
                                                          const float* __restrict__ part_ml, int S, int Dv, float sink,
-                                                         int H, const T* __restrict__ gate, int gate_stride) {
+                                                         int H, const T* __restrict__ gate, int gate_stride,
+                                                         float out_scale, int out_stride, int out_off) {
   const size_t rh = blockIdx.x;
   const int lane = threadIdx.x;
   float M = kNeg;
@@ -197,9 +202,9 @@ __global__ void __launch_bounds__(64) gqa_combine_kernel(T* __restrict__ out, co
   for (int col = lane; col < Dv; col += 64) {
     float acc = 0.f;
     for (int s = 0; s < S; ++s) acc += part_o[(rh * S + s) * Dv + col] * __expf(part_ml[(rh * S + s) * 2] - M);
-    float v = acc * inv;
+    float v = acc * inv * out_scale;
     if (gate) v *= 1.0f / (1.0f + __expf(-DT<T>::load(gate + (rh / H) * gate_stride + (rh % H) * Dv + col)));
-    DT<T>::store(out + rh * Dv + col, v);
+    DT<T>::store(out + (rh / H) * out_stride + out_off + (rh % H) * Dv + col, v);
   }
 }
 
@@ -220,7 +225,8 @@ int launch_gqa_attention(void* out, const void* q, const void* kc, const void* v
                          const int* cu_q, const int* start_pos, const int* tiles, int n_tiles, const float* temp,
                          float* part_o, float* part_ml, int T, int H, int G, int Dk, int Dv, int BS, int max_blocks,
                          int rows, int num_splits, float scale, float sink, int window, const float* slopes,
-                         const void* gate, int gate_stride, int layout, bool bf, hipStream_t stream) {
+                         const void* gate, int gate_stride, int layout, float softcap, float out_scale, int out_stride,
+                         int out_off, bool bf, hipStream_t stream) {
   if (n_tiles <= 0 || T <= 0) return 0;
   const int KT = gqa_key_tile(Dk, Dv);
   if (KT == 0 || Dv > 256 || Dk > 256 || H % G) return -1;
@@ -244,7 +250,8 @@ int launch_gqa_attention(void* out, const void* q, const void* kc, const void* v
       return -3;                                                                                                     \
     kern<<<grid, 256, shm, stream>>>((TT*)out, (const TT*)q, (const TT*)kc, (const TT*)vc, block_tables, cu_q,      \
                                      start_pos, tiles, temp, part_o, part_ml, H, G, Dk, Dv, BS, max_blocks, rows,   \
-                                     KT, hchunks, scale, sink, window, slopes, (const TT*)gate, gate_stride, layout); \
+                                     KT, hchunks, scale, sink, window, slopes, (const TT*)gate, gate_stride, layout, \
+                                     softcap, out_scale, out_stride, out_off);                                      \
   } while (0)
   if (bf) {
     if (dvl == 1) RT_GQA(uint16_t, 1); else if (dvl == 2) RT_GQA(uint16_t, 2); else RT_GQA(uint16_t, 4);
@@ -255,9 +262,11 @@ int launch_gqa_attention(void* out, const void* q, const void* kc, const void* v
 #undef RT_GQA2
   if (num_splits > 1) {
     if (bf) gqa_combine_kernel<uint16_t><<<T * H, 64, 0, stream>>>((uint16_t*)out, part_o, part_ml, num_splits, Dv, sink, H,
-                                                                   (const uint16_t*)gate, gate_stride);
+                                                                   (const uint16_t*)gate, gate_stride, out_scale,
+                                                                   out_stride, out_off);
     else gqa_combine_kernel<float><<<T * H, 64, 0, stream>>>((float*)out, part_o, part_ml, num_splits, Dv, sink, H,
-                                                             (const float*)gate, gate_stride);
+                                                             (const float*)gate, gate_stride, out_scale, out_stride,
+                                                             out_off);
   }
   return 0;
 }

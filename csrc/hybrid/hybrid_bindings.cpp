@@ -35,7 +35,8 @@ int launch_gqa_attention(void* out, const void* q, const void* kc, const void* v
                          const int* cu_q, const int* start_pos, const int* tiles, int n_tiles, const float* temp,
                          float* part_o, float* part_ml, int T, int H, int G, int Dk, int Dv, int BS, int max_blocks,
                          int rows, int num_splits, float scale, float sink, int window, const float* slopes,
-                         const void* gate, int gate_stride, int layout, bool bf, hipStream_t stream);
+                         const void* gate, int gate_stride, int layout, float softcap, float out_scale, int out_stride,
+                         int out_off, bool bf, hipStream_t stream);
 int wkv_scan_chunk();
 int launch_wkv_scan(void* out, const void* r, const void* k, const void* v, const void* g, const void* lw, int stride,
                     int lw_stride, const float* w0, const float* u, const float* norm_w, float* state, const int* cu_q,
@@ -46,7 +47,36 @@ void launch_xielu(void* out, const void* a, const float* bias, int64_t rows, int
 void launch_silu_glu(void* out, const void* gu, int64_t rows, int F, bool bf, hipStream_t stream);
 int launch_topk_softmax(int* idx, float* wt, const float* logits, int T, int E, int top, hipStream_t stream);
 int launch_moe_rows(void* out, float* hid, const void* h, const void* wgu, const void* wd, const int* idx,
-                    const float* wt, int T, int W, int F, int top, bool bf, hipStream_t stream);
+                    const float* wt, int T, int W, int F, int top, int act, bool bf, hipStream_t stream);
+void launch_canon_add(void* h, float* xs, const float* x, const void* y, const void* y2, const float* nw, float eps,
+                      const float* cw, float* state, int sub, int nsub, const int* row_seq, const int64_t* positions,
+                      const int* start_pos, const int* slots, int T, int W, int taps, int keep, bool out_bf, bool y_bf,
+                      bool shift_state, hipStream_t stream);
+void launch_conv_state(const void* x, int stride, int col_off, int C, float* state, int sub, int nsub, int keep,
+                       const int* cu_q, const int* start_pos, const int* slots, int S, bool bf, hipStream_t stream);
+int launch_qkv_prep_wide(void* q, const void* proj, int stride, int q_off, int k_off, int v_off, bool v_from_k,
+                         const float* qb, const float* kb, const float* qw, const float* kw, const float* freq, int R,
+                         float mag, const float* vfreq, float eps, const int64_t* positions, void* kc, void* vc,
+                         const int64_t* slot_mapping, int T, int H, int G, int Dk, int Dv, int BS, bool bf,
+                         hipStream_t stream);
+void launch_turn_back(void* out, int out_stride, int out_off, const void* o, int T, int H, int E,
+                      const int64_t* positions, const float* vfreq, float scale, bool bf, hipStream_t stream);
+void launch_silu_cols(float* out, const void* proj, int stride, int off, int n, int T, bool bf, hipStream_t stream);
+void launch_relu2(void* out, const void* a, int64_t total, bool bf, hipStream_t stream);
+void launch_removal_prep(float* out, const void* proj, int stride, int r_off, int k_off, int v_off, int a_off,
+                         const void* lw, const float* w0, const float* ab, int T, int A, int D, bool bf,
+                         hipStream_t stream);
+int launch_delta_prep(float* five, float* vout, const void* proj, int stride, int q_off, int b_off, int a_off,
+                      const float* cw, float* state, const float* neg_rate, const float* dt_bias, int T, int A, int G,
+                      int D, int E, int taps, int keep, const int* row_seq, const int64_t* positions,
+                      const int* start_pos, const int* slots, bool shift_state, bool bf, hipStream_t stream);
+void launch_head_norm_gate(void* out, int out_stride, int out_off, const float* o, const float* w, int wmod, int span,
+                           const void* gate, int gate_stride, int gate_off, int act, float eps, float scale, int T, int C,
+                           bool out_bf, bool gate_bf, hipStream_t stream);
+int launch_state_scan(float* out, const float* q, const float* k, const float* v, const float* w, const float* a,
+                      const float* b, int sq, int sk, int sv, int sw, int sa, int sb, const float* decay, float* state,
+                      const int* cu_q, const int* start_pos, const int* slots, int S, int A, int D, int E,
+                      hipStream_t stream);
 
 namespace {
 
@@ -165,7 +195,8 @@ void gqa_attention(torch::Tensor out, torch::Tensor q, torch::Tensor kc, torch::
                    torch::Tensor cu_q, torch::Tensor start_pos, torch::Tensor tiles, c10::optional<torch::Tensor> temp,
                    double scale, double sink, int64_t rows, int64_t num_splits, c10::optional<torch::Tensor> part_o,
                    c10::optional<torch::Tensor> part_ml, int64_t window, c10::optional<torch::Tensor> slopes,
-                   c10::optional<torch::Tensor> gate, int64_t gate_off, int64_t layout) {
+                   c10::optional<torch::Tensor> gate, int64_t gate_off, int64_t layout, double softcap, double out_scale,
+                   int64_t out_off) {
   chk_act(out, "out"); chk_act(q, "q"); chk_act(kc, "k_cache"); chk_act(vc, "v_cache");
   TORCH_CHECK(out.scalar_type() == q.scalar_type() && kc.scalar_type() == q.scalar_type() &&
               vc.scalar_type() == q.scalar_type(), "gqa_attention: one dtype for q, the cache and out");
@@ -176,7 +207,8 @@ void gqa_attention(torch::Tensor out, torch::Tensor q, torch::Tensor kc, torch::
   TORCH_CHECK(kc.size(3) == Dk && vc.size(0) == kc.size(0) && vc.size(1) == G && vc.size(layout ? 3 : 2) == BS &&
               H % G == 0, "gqa_attention: cache shapes");
   TORCH_CHECK(layout == 0 || Dk % 32 == 0, "gqa_attention: the matrix-core key layout needs dim % 32 == 0");
-  TORCH_CHECK(out.size(0) == T && out.size(1) == H * Dv, "gqa_attention: out [T, H * Dv]");
+  TORCH_CHECK(out.size(0) == T && out_off >= 0 && out_off + H * Dv <= out.size(1) && softcap >= 0,
+              "gqa_attention: out [T, >= out_off + H * Dv]");
   chk_i32(block_tables, "block_tables"); chk_i32(cu_q, "cu_q"); chk_i32(start_pos, "start_pos", cu_q.numel() - 1);
   chk_i32(tiles, "tiles");
   TORCH_CHECK(block_tables.dim() == 2 && block_tables.size(0) == start_pos.numel(), "gqa_attention: block_tables [S, n]");
@@ -213,7 +245,8 @@ void gqa_attention(torch::Tensor out, torch::Tensor q, torch::Tensor kc, torch::
   int rc = launch_gqa_attention(out.data_ptr(), q.data_ptr(), kc.data_ptr(), vc.data_ptr(), block_tables.data_ptr<int>(),
                                 cu_q.data_ptr<int>(), start_pos.data_ptr<int>(), tiles.data_ptr<int>(), tiles.size(0), tp,
                                 po, pml, T, H, G, Dk, Dv, BS, block_tables.size(1), rows, num_splits, (float)scale,
-                                (float)sink, (int)window, sl, gp, (int)gstride, (int)layout, is_bf(q), cur());
+                                (float)sink, (int)window, sl, gp, (int)gstride, (int)layout, (float)softcap,
+                                (float)out_scale, (int)out.size(1), (int)out_off, is_bf(q), cur());
   TORCH_CHECK(rc == 0, "gqa_attention: unsupported shape (code ", rc, ": -1 head sizes beyond 256 or the LDS tile, "
               "-2 rows per tile, -3 LDS size refused)");
 }
@@ -344,19 +377,252 @@ void topk_softmax(torch::Tensor idx, torch::Tensor wt, torch::Tensor logits) {
 
 // wgu [E, 2F, W] (gate rows, then up rows), wd [E, W, F]; idx / wt [T, top]; hid fp32 [T, top, F] scratch
 void moe_rows(torch::Tensor out, torch::Tensor hid, torch::Tensor h, torch::Tensor wgu, torch::Tensor wd, torch::Tensor idx,
-              torch::Tensor wt) {
+              torch::Tensor wt, int64_t act) {
   chk_act(out, "out"); chk_act(h, "h"); chk_act(wgu, "wgu"); chk_act(wd, "wd"); chk_f32(hid, "hid");
   TORCH_CHECK(h.dim() == 2 && wgu.dim() == 3 && wd.dim() == 3 && idx.dim() == 2, "moe_rows: ranks");
   const int64_t T = h.size(0), W = h.size(1), E = wgu.size(0), F = wd.size(2), top = idx.size(1);
-  TORCH_CHECK(wgu.size(1) == 2 * F && wgu.size(2) == W && wd.size(0) == E && wd.size(1) == W && idx.size(0) == T &&
+  TORCH_CHECK((act == 0 || act == 1) && wgu.size(1) == (act ? 1 : 2) * F && wgu.size(2) == W && wd.size(0) == E && wd.size(1) == W && idx.size(0) == T &&
               out.sizes() == h.sizes(), "moe_rows: shapes");
   TORCH_CHECK(out.scalar_type() == h.scalar_type() && wgu.scalar_type() == h.scalar_type() &&
               wd.scalar_type() == h.scalar_type(), "moe_rows: one dtype");
   chk_i32(idx, "idx"); chk_f32(wt, "wt", T * top);
   TORCH_CHECK(hid.numel() >= T * top * F, "moe_rows: scratch too small");
   int rc = launch_moe_rows(out.data_ptr(), hid.data_ptr<float>(), h.data_ptr(), wgu.data_ptr(), wd.data_ptr(),
-                           idx.data_ptr<int>(), wt.data_ptr<float>(), T, W, F, top, is_bf(h), cur());
+                           idx.data_ptr<int>(), wt.data_ptr<float>(), T, W, F, top, (int)act, is_bf(h), cur());
   TORCH_CHECK(rc == 0, "moe_rows: a row does not fit the LDS");
+}
+
+using OptT = c10::optional<torch::Tensor>;
+
+const float* opt_f32(const OptT& t, const char* name, int64_t n) {
+  if (!t.has_value()) return nullptr;
+  chk_f32(*t, name, n);
+  return t->data_ptr<float>();
+}
+
+// rows [T] / spans [S] of a batch, checked against each other
+void chk_rows(const torch::Tensor& row_seq, const torch::Tensor& positions, const torch::Tensor& start_pos,
+              const torch::Tensor& slots, int64_t T, int64_t n_slots) {
+  chk_i32(row_seq, "row_seq", T);
+  chk_i64(positions, "positions", T);
+  chk_i32(start_pos, "start_pos");
+  chk_i32(slots, "slots", start_pos.numel());
+  (void)n_slots;
+}
+
+void canon_add(OptT h, torch::Tensor xs, torch::Tensor x, OptT y, OptT y2, OptT nw, double eps, OptT cw, OptT state,
+               int64_t sub, torch::Tensor row_seq, torch::Tensor positions, torch::Tensor start_pos, torch::Tensor slots,
+               bool shift_state) {
+  chk_f32(x, "x"); chk_f32(xs, "xs", x.numel());
+  TORCH_CHECK(x.dim() == 2, "canon_add: x [T, W]");
+  const int64_t T = x.size(0), W = x.size(1);
+  if (T == 0 || (!y.has_value() && !cw.has_value())) return;
+  bool y_bf = false;
+  if (y.has_value()) {
+    chk_act(*y, "y");
+    TORCH_CHECK(y->numel() == x.numel() && nw.has_value() && xs.data_ptr() != x.data_ptr(),
+                "canon_add: y [T, W] needs the norm weight and an output of its own");
+    y_bf = is_bf(*y);
+    if (y2.has_value()) {
+      chk_act(*y2, "y2");
+      TORCH_CHECK(y2->numel() == x.numel() && y2->scalar_type() == y->scalar_type(), "canon_add: y2 like y");
+    }
+  } else {
+    TORCH_CHECK(xs.data_ptr() == x.data_ptr() && !y2.has_value(), "canon_add: without y the residual is x itself");
+  }
+  int taps = 0, keep = 0, nsub = 1;
+  void* hp = nullptr;
+  bool out_bf = false;
+  if (cw.has_value()) {
+    chk_f32(*cw, "conv_w");
+    TORCH_CHECK(cw->dim() == 2 && cw->size(0) == W && cw->size(1) >= 1 && cw->size(1) <= 16, "canon_add: conv_w [W, taps <= 16]");
+    taps = (int)cw->size(1);
+    TORCH_CHECK(h.has_value() && state.has_value(), "canon_add: the convolution needs h and the state");
+    chk_act(*h, "h");
+    TORCH_CHECK(h->numel() == x.numel(), "canon_add: h [T, W]");
+    chk_f32(*state, "state");
+    TORCH_CHECK(state->dim() == 4 && state->size(3) == W && state->size(2) >= std::max(taps - 1, 1) && sub >= 0 &&
+                sub < state->size(1), "canon_add: state [slots, subs, taps - 1, W]");
+    TORCH_CHECK(state->size(2) == std::max(taps - 1, 1), "canon_add: state rows");
+    keep = (int)state->size(2);
+    nsub = (int)state->size(1);
+    chk_rows(row_seq, positions, start_pos, slots, T, state->size(0));
+    hp = h->data_ptr();
+    out_bf = is_bf(*h);
+  }
+  launch_canon_add(hp, xs.data_ptr<float>(), x.data_ptr<float>(), y.has_value() ? y->data_ptr() : nullptr,
+                   y2.has_value() ? y2->data_ptr() : nullptr, opt_f32(nw, "norm_w", W), (float)eps,
+                   cw.has_value() ? cw->data_ptr<float>() : nullptr, cw.has_value() ? state->data_ptr<float>() : nullptr,
+                   (int)sub, nsub, cw.has_value() ? row_seq.data_ptr<int>() : nullptr,
+                   cw.has_value() ? positions.data_ptr<int64_t>() : nullptr,
+                   cw.has_value() ? start_pos.data_ptr<int>() : nullptr, cw.has_value() ? slots.data_ptr<int>() : nullptr,
+                   (int)T, (int)W, taps, keep, out_bf, y_bf, shift_state, cur());
+}
+
+void conv_state_update(torch::Tensor x, int64_t col_off, int64_t C, torch::Tensor state, int64_t sub, torch::Tensor cu_q,
+                       torch::Tensor start_pos, torch::Tensor slots) {
+  chk_act(x, "x"); chk_f32(state, "state");
+  TORCH_CHECK(x.dim() == 2 && col_off >= 0 && col_off + C <= x.size(1), "conv_state_update: columns");
+  TORCH_CHECK((state.dim() == 4 || state.dim() == 3) && state.size(-1) == C && state.size(-2) <= 16,
+              "conv_state_update: state [slots, (subs,) keep, C]");
+  const int nsub = state.dim() == 4 ? (int)state.size(1) : 1;
+  TORCH_CHECK(sub >= 0 && sub < nsub, "conv_state_update: sub");
+  const int64_t S = cu_q.numel() - 1;
+  chk_i32(cu_q, "cu_q"); chk_i32(start_pos, "start_pos", S); chk_i32(slots, "slots", S);
+  launch_conv_state(x.data_ptr(), (int)x.size(1), (int)col_off, (int)C, state.data_ptr<float>(), (int)sub, nsub,
+                    (int)state.size(-2), cu_q.data_ptr<int>(), start_pos.data_ptr<int>(), slots.data_ptr<int>(), (int)S,
+                    is_bf(x), cur());
+}
+
+void qkv_prep_wide(torch::Tensor q, torch::Tensor proj, int64_t q_off, int64_t k_off, int64_t v_off, bool v_from_k,
+                   OptT qb, OptT kb, torch::Tensor qw, torch::Tensor kw, OptT freq, double mag, OptT vfreq, double eps,
+                   torch::Tensor positions, torch::Tensor kc, torch::Tensor vc, torch::Tensor slot_mapping) {
+  chk_act(q, "q"); chk_act(proj, "proj"); chk_act(kc, "k_cache"); chk_act(vc, "v_cache");
+  TORCH_CHECK(q.dim() == 3 && proj.dim() == 2 && kc.dim() == 4 && vc.dim() == 4, "qkv_prep_wide: ranks");
+  TORCH_CHECK(q.scalar_type() == proj.scalar_type() && kc.scalar_type() == proj.scalar_type() &&
+              vc.scalar_type() == proj.scalar_type(), "qkv_prep_wide: one dtype");
+  const int64_t T = q.size(0), H = q.size(1), Dk = q.size(2), G = kc.size(1), BS = kc.size(2), Dv = vc.size(3), N = proj.size(1);
+  TORCH_CHECK(proj.size(0) == T && kc.size(3) == Dk && vc.size(0) == kc.size(0) && vc.size(1) == G && vc.size(2) == BS,
+              "qkv_prep_wide: shapes");
+  TORCH_CHECK(q_off >= 0 && q_off + H * Dk <= N && k_off >= 0 && k_off + G * Dk <= N, "qkv_prep_wide: q / k columns");
+  TORCH_CHECK(v_from_k ? Dv == Dk : (v_off >= 0 && v_off + G * Dv <= N), "qkv_prep_wide: value columns");
+  chk_f32(qw, "q_w", H * Dk); chk_f32(kw, "k_w", G * Dk);
+  int R = 0;
+  if (freq.has_value()) {
+    chk_f32(*freq, "freq");
+    R = (int)freq->numel();
+    TORCH_CHECK(2 * R <= Dk, "qkv_prep_wide: rotated entries beyond the head");
+  }
+  if (vfreq.has_value()) {
+    chk_f32(*vfreq, "vfreq", Dv / 2);
+    TORCH_CHECK(Dv % 2 == 0 && !v_from_k, "qkv_prep_wide: turned values need an even vdim and a value projection");
+  }
+  chk_i64(positions, "positions", T); chk_i64(slot_mapping, "slot_mapping", T);
+  int rc = launch_qkv_prep_wide(q.data_ptr(), proj.data_ptr(), (int)N, (int)q_off, (int)k_off, (int)v_off, v_from_k,
+                                opt_f32(qb, "q_bias", H * Dk), opt_f32(kb, "k_bias", G * Dk), qw.data_ptr<float>(),
+                                kw.data_ptr<float>(), freq.has_value() ? freq->data_ptr<float>() : nullptr, R, (float)mag,
+                                vfreq.has_value() ? vfreq->data_ptr<float>() : nullptr, (float)eps,
+                                positions.data_ptr<int64_t>(), kc.data_ptr(), vc.data_ptr(),
+                                slot_mapping.data_ptr<int64_t>(), (int)T, (int)H, (int)G, (int)Dk, (int)Dv, (int)BS,
+                                is_bf(proj), cur());
+  TORCH_CHECK(rc == 0, "qkv_prep_wide: the query and key rows do not fit the LDS (code ", rc, ")");
+}
+
+void turn_back(torch::Tensor out, int64_t out_off, torch::Tensor o, int64_t H, torch::Tensor positions,
+               torch::Tensor vfreq, double scale) {
+  chk_act(out, "out"); chk_act(o, "o");
+  TORCH_CHECK(out.dim() == 2 && o.dim() == 2 && out.size(0) == o.size(0) && out.scalar_type() == o.scalar_type() &&
+              H >= 1 && o.size(1) % H == 0 && out_off >= 0 && out_off + o.size(1) <= out.size(1), "turn_back: shapes");
+  const int64_t E = o.size(1) / H;
+  TORCH_CHECK(E % 2 == 0, "turn_back: even head size");
+  chk_f32(vfreq, "vfreq", E / 2); chk_i64(positions, "positions", o.size(0));
+  launch_turn_back(out.data_ptr(), (int)out.size(1), (int)out_off, o.data_ptr(), (int)o.size(0), (int)H, (int)E,
+                   positions.data_ptr<int64_t>(), vfreq.data_ptr<float>(), (float)scale, is_bf(o), cur());
+}
+
+void silu_cols(torch::Tensor out, torch::Tensor proj, int64_t off) {
+  chk_f32(out, "out"); chk_act(proj, "proj");
+  TORCH_CHECK(out.dim() == 2 && proj.dim() == 2 && out.size(0) == proj.size(0) && off >= 0 &&
+              off + out.size(1) <= proj.size(1), "silu_cols: columns");
+  launch_silu_cols(out.data_ptr<float>(), proj.data_ptr(), (int)proj.size(1), (int)off, (int)out.size(1),
+                   (int)out.size(0), is_bf(proj), cur());
+}
+
+void relu2(torch::Tensor out, torch::Tensor a) {
+  chk_act(out, "out"); chk_act(a, "a");
+  TORCH_CHECK(out.numel() == a.numel() && out.scalar_type() == a.scalar_type(), "relu2: out like a");
+  launch_relu2(out.data_ptr(), a.data_ptr(), a.numel(), is_bf(a), cur());
+}
+
+void removal_prep(torch::Tensor out, torch::Tensor proj, int64_t r_off, int64_t k_off, int64_t v_off, int64_t a_off,
+                  torch::Tensor lw, torch::Tensor w0, torch::Tensor ab, int64_t A) {
+  chk_f32(out, "out"); chk_act(proj, "proj"); chk_act(lw, "lw");
+  TORCH_CHECK(out.dim() == 3 && out.size(0) == 6 && proj.dim() == 2 && out.size(1) == proj.size(0) && A >= 1 &&
+              out.size(2) % A == 0, "removal_prep: out [6, T, A * D]");
+  const int64_t T = proj.size(0), n = out.size(2), N = proj.size(1);
+  for (int64_t o : {r_off, k_off, v_off, a_off}) TORCH_CHECK(o >= 0 && o + n <= N, "removal_prep: columns");
+  TORCH_CHECK(lw.dim() == 2 && lw.size(0) == T && lw.size(1) == n && lw.scalar_type() == proj.scalar_type(),
+              "removal_prep: lw [T, A * D] of proj's dtype");
+  chk_f32(w0, "w0", n); chk_f32(ab, "a_bias", n);
+  launch_removal_prep(out.data_ptr<float>(), proj.data_ptr(), (int)N, (int)r_off, (int)k_off, (int)v_off, (int)a_off,
+                      lw.data_ptr(), w0.data_ptr<float>(), ab.data_ptr<float>(), (int)T, (int)A, (int)(n / A),
+                      is_bf(proj), cur());
+}
+
+void delta_prep(torch::Tensor five, torch::Tensor vout, torch::Tensor proj, int64_t q_off, int64_t b_off, int64_t a_off,
+                torch::Tensor cw, torch::Tensor state, torch::Tensor neg_rate, torch::Tensor dt_bias, int64_t A, int64_t G,
+                int64_t D, int64_t E, torch::Tensor row_seq, torch::Tensor positions, torch::Tensor start_pos,
+                torch::Tensor slots, bool shift_state) {
+  chk_act(proj, "proj");
+  TORCH_CHECK(proj.dim() == 2 && A >= 1 && G >= 1 && A % G == 0 && D >= 1 && E >= 1, "delta_prep: sizes");
+  const int64_t T = proj.size(0), N = proj.size(1), C = 2 * G * D + A * E;
+  chk_f32(five, "five", 5 * T * A * D); chk_f32(vout, "v", T * A * E);
+  TORCH_CHECK(q_off >= 0 && q_off + C <= N && b_off >= 0 && b_off + A <= N && a_off >= 0 && a_off + A <= N,
+              "delta_prep: columns");
+  chk_f32(cw, "conv_w");
+  TORCH_CHECK(cw.dim() == 2 && cw.size(0) == C && cw.size(1) >= 1 && cw.size(1) <= 16, "delta_prep: conv_w [C, taps <= 16]");
+  const int taps = (int)cw.size(1);
+  chk_f32(state, "state");
+  TORCH_CHECK(state.dim() == 3 && state.size(2) == C && state.size(1) == std::max(taps - 1, 1),
+              "delta_prep: state [slots, taps - 1, C]");
+  chk_f32(neg_rate, "neg_rate", A); chk_f32(dt_bias, "dt_bias", A);
+  chk_rows(row_seq, positions, start_pos, slots, T, state.size(0));
+  int rc = launch_delta_prep(five.data_ptr<float>(), vout.data_ptr<float>(), proj.data_ptr(), (int)N, (int)q_off,
+                             (int)b_off, (int)a_off, cw.data_ptr<float>(), state.data_ptr<float>(),
+                             neg_rate.data_ptr<float>(), dt_bias.data_ptr<float>(), (int)T, (int)A, (int)G, (int)D, (int)E,
+                             taps, (int)state.size(1), row_seq.data_ptr<int>(), positions.data_ptr<int64_t>(),
+                             start_pos.data_ptr<int>(), slots.data_ptr<int>(), shift_state, is_bf(proj), cur());
+  TORCH_CHECK(rc == 0, "delta_prep: a row does not fit the LDS (code ", rc, ")");
+}
+
+// an fp32 row stream [T, >= A * n] with unit column stride: pointer and row stride
+const float* stream_of(const OptT& t, const char* name, int64_t T, int64_t n, int& stride) {
+  stride = 0;
+  if (!t.has_value()) return nullptr;
+  TORCH_CHECK(t->is_cuda() && t->scalar_type() == torch::kFloat32 && t->dim() == 2 && t->size(0) == T &&
+              t->size(1) == n && (t->size(1) == 1 || t->stride(1) == 1) && t->stride(0) >= n, name,
+              " must be an fp32 [T, heads * size] GPU tensor with unit column stride");
+  stride = (int)t->stride(0);
+  return t->data_ptr<float>();
+}
+
+void state_scan(torch::Tensor out, torch::Tensor q, torch::Tensor k, torch::Tensor v, OptT w, OptT a, OptT b, OptT decay,
+                torch::Tensor state, torch::Tensor cu_q, torch::Tensor start_pos, torch::Tensor slots, int64_t A, int64_t D,
+                int64_t E) {
+  TORCH_CHECK(A >= 1 && D >= 1 && D <= 256 && E >= 1, "state_scan: heads, dim <= 256, vdim");
+  TORCH_CHECK(q.dim() == 2, "state_scan: q [T, A * D]");
+  const int64_t T = q.size(0), S = cu_q.numel() - 1;
+  chk_f32(out, "out", T * A * E);
+  int sq, sk, sv, sw, sa, sb;
+  const float* qp = stream_of(q, "q", T, A * D, sq);
+  const float* kp = stream_of(k, "k", T, A * D, sk);
+  const float* vp = stream_of(v, "v", T, A * E, sv);
+  const float* wp = stream_of(w, "w", T, A * D, sw);
+  const float* ap = stream_of(a, "a", T, A * D, sa);
+  const float* bp = stream_of(b, "b", T, A * D, sb);
+  TORCH_CHECK(a.has_value() == b.has_value(), "state_scan: a and b come together");
+  TORCH_CHECK(w.has_value() != decay.has_value(), "state_scan: either a decay stream or a constant per head");
+  chk_f32(state, "state");
+  TORCH_CHECK(state.dim() == 2 && state.size(1) == A * D * E, "state_scan: state [slots, A * E * D]");
+  chk_i32(cu_q, "cu_q"); chk_i32(start_pos, "start_pos", S); chk_i32(slots, "slots", S);
+  int rc = launch_state_scan(out.data_ptr<float>(), qp, kp, vp, wp, ap, bp, sq, sk, sv, sw, sa, sb,
+                             opt_f32(decay, "decay", A), state.data_ptr<float>(), cu_q.data_ptr<int>(),
+                             start_pos.data_ptr<int>(), slots.data_ptr<int>(), (int)S, (int)A, (int)D, (int)E, cur());
+  TORCH_CHECK(rc == 0, "state_scan: unsupported shape (code ", rc, ")");
+}
+
+void head_norm_gate(torch::Tensor out, int64_t out_off, torch::Tensor o, torch::Tensor w, int64_t span, torch::Tensor gate,
+                    int64_t gate_off, int64_t act, double eps, double scale) {
+  chk_act(out, "out"); chk_f32(o, "o"); chk_act(gate, "gate"); chk_f32(w, "norm_w");
+  TORCH_CHECK(out.dim() == 2 && o.dim() == 2 && gate.dim() == 2 && out.size(0) == o.size(0) && gate.size(0) == o.size(0),
+              "head_norm_gate: ranks");
+  const int64_t T = o.size(0), C = o.size(1);
+  TORCH_CHECK(span >= 1 && C % span == 0 && (w.numel() == C || w.numel() == span), "head_norm_gate: span / weight");
+  TORCH_CHECK(out_off >= 0 && out_off + C <= out.size(1) && gate_off >= 0 && gate_off + C <= gate.size(1),
+              "head_norm_gate: columns");
+  launch_head_norm_gate(out.data_ptr(), (int)out.size(1), (int)out_off, o.data_ptr<float>(), w.data_ptr<float>(),
+                        (int)w.numel(), (int)span, gate.data_ptr(), (int)gate.size(1), (int)gate_off, (int)act, (float)eps,
+                        (float)scale, (int)T, (int)C, is_bf(out), is_bf(gate), cur());
 }
 
 }  // namespace
@@ -376,7 +642,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("block_tables"), py::arg("cu_q"), py::arg("start_pos"), py::arg("tiles"), py::arg("temp"), py::arg("scale"),
         py::arg("sink"), py::arg("rows"), py::arg("num_splits"), py::arg("part_o"), py::arg("part_ml"),
         py::arg("window") = 0, py::arg("slopes") = py::none(), py::arg("gate") = py::none(), py::arg("gate_off") = 0,
-        py::arg("layout") = 0);
+        py::arg("layout") = 0, py::arg("softcap") = 0.0, py::arg("out_scale") = 1.0, py::arg("out_off") = 0);
   m.def("mingru_scan", &mingru_scan, py::arg("out"), py::arg("proj"), py::arg("z_off"), py::arg("x_off"), py::arg("g_off"),
         py::arg("bz"), py::arg("bx"), py::arg("state"), py::arg("cu_q"), py::arg("start_pos"), py::arg("slots"),
         py::arg("chunks") = py::none(), py::arg("seq_chunk0") = py::none(), py::arg("ws") = py::none());
@@ -391,6 +657,17 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("xielu", &xielu);
   m.def("silu_glu", &silu_glu);
   m.def("topk_softmax", &topk_softmax);
-  m.def("moe_rows", &moe_rows);
+  m.def("moe_rows", &moe_rows, py::arg("out"), py::arg("hid"), py::arg("h"), py::arg("wgu"), py::arg("wd"), py::arg("idx"),
+        py::arg("wt"), py::arg("act") = 0);
   m.def("limited_glu", &limited_glu);
+  m.def("canon_add", &canon_add);
+  m.def("conv_state_update", &conv_state_update);
+  m.def("qkv_prep_wide", &qkv_prep_wide);
+  m.def("turn_back", &turn_back);
+  m.def("silu_cols", &silu_cols);
+  m.def("relu2", &relu2);
+  m.def("removal_prep", &removal_prep);
+  m.def("delta_prep", &delta_prep);
+  m.def("state_scan", &state_scan);
+  m.def("head_norm_gate", &head_norm_gate);
 }

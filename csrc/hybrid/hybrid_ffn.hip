@@ -151,22 +151,34 @@ constexpr int kMoeWaves = 4;
 constexpr int kMoeRows = 4;         // output entries a wave computes together
 constexpr int kMoeBlock = kMoeWaves * kMoeRows;
 
-// grid (T * top, blocks of kMoeBlock over F); wgu [E, 2F, W] = (gate | up) rows of every expert
+// grid (T * top, blocks of kMoeBlock over F); wgu [E, 2F, W] = (gate | up) rows of every expert;
+// act 1: experts without a gate, wgu [E, F, W], hidden = relu(up)^2
 template <typename T>
 __global__ void __launch_bounds__(64 * kMoeWaves) moe_gate_up_kernel(float* __restrict__ hid, const T* __restrict__ h,
                                                                      const T* __restrict__ wgu,
-                                                                     const int* __restrict__ idx, int W, int F, int top) {
+                                                                     const int* __restrict__ idx, int W, int F, int top,
+                                                                     int act) {
   extern __shared__ float xs[];
   const int pair = blockIdx.x, t = pair / top;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (int c = threadIdx.x; c < W; c += blockDim.x) xs[c] = DT<T>::load(h + (size_t)t * W + c);
   __syncthreads();
-  const T* we = wgu + (size_t)idx[pair] * 2 * F * W;
+  const T* we = wgu + (size_t)idx[pair] * (act ? 1 : 2) * F * W;
   const int f = blockIdx.y * kMoeBlock + wave * kMoeRows;
   const int ok = min(kMoeRows, F - f);
   if (ok <= 0) return;
   float gv[kMoeRows], uv[kMoeRows];
   dot_rows<kMoeRows>(we + (size_t)f * W, (size_t)W, ok, xs, W, lane, gv);
+  if (act) {
+    if (lane < ok) {
+      float u = 0.f;
+#pragma unroll
+      for (int r = 0; r < kMoeRows; ++r)
+        if (r == lane) u = fmaxf(gv[r], 0.f);
+      hid[(size_t)pair * F + f + lane] = u * u;
+    }
+    return;
+  }
   dot_rows<kMoeRows>(we + (size_t)(F + f) * W, (size_t)W, ok, xs, W, lane, uv);
   if (lane < ok) {
     float g = 0.f, u = 0.f;
@@ -239,7 +251,7 @@ int launch_topk_softmax(int* idx, float* wt, const float* logits, int T, int E, 
 }
 
 int launch_moe_rows(void* out, float* hid, const void* h, const void* wgu, const void* wd, const int* idx,
-                    const float* wt, int T, int W, int F, int top, bool bf, hipStream_t stream) {
+                    const float* wt, int T, int W, int F, int top, int act, bool bf, hipStream_t stream) {
   if (T <= 0) return 0;
   const size_t shm1 = sizeof(float) * (size_t)W, shm2 = sizeof(float) * (size_t)top * F;
   if (shm1 > 150 * 1024 || shm2 > 150 * 1024) return -1;
@@ -256,7 +268,7 @@ int launch_moe_rows(void* out, float* hid, const void* h, const void* wgu, const
     if (shm2 > 48 * 1024 &&                                                                                            \
         hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm2) != hipSuccess)     \
       return -2;                                                                                                       \
-    k1<<<g1, 64 * kMoeWaves, shm1, stream>>>(hid, (const TT*)h, (const TT*)wgu, idx, W, F, top);                       \
+    k1<<<g1, 64 * kMoeWaves, shm1, stream>>>(hid, (const TT*)h, (const TT*)wgu, idx, W, F, top, act);                    \
     k2<<<g2, 64 * kMoeWaves, shm2, stream>>>((TT*)out, hid, (const TT*)wd, idx, wt, W, F, top);                        \
   } while (0)
   if (bf) RT_MOE(uint16_t); else RT_MOE(float);
