@@ -114,7 +114,7 @@ def parse():
                         "JSON (parallel/costmodel.py default_calibration, $ROUNDTABLE_CALIBRATION)")
     p.add_argument("--arch-compare", default="",
                    help="instead of the headline workload: prefill and decode throughput of model pairs "
-                        "'a:b,c:d' (e.g. mupulorn-8b:llama3-8b,goganex-8b:llama3-8b,retuvik-1b:llama3.2-1b), each model with "
+                        "'a:b,c:d' (e.g. mupulorn-8b:llama3-8b,goganex-8b:llama3-8b,retuvik-1b:llama3.2-1b,ledinex-0.5b:retuvik-0.5b), each model with "
                         "--compare-layers layers and random weights, through the same engine entry points; "
                         "prints one JSON line per model")
     p.add_argument("--retuvik-large", action="store_true",
@@ -183,8 +183,8 @@ def _arch_compare(args) -> int:
             t_dec = time.perf_counter() - t0
             cfg = eng.cfg
             print(json.dumps({"metric": "arch compare", "model": name, "layers": L, "params_per_layer_M":
-                              round((cfg.n_params() - (1 if cfg.tie_embeddings and cfg.layers is None else 2)
-                                     * cfg.vocab * cfg.hidden) / L / 1e6, 1),
+                              round((cfg.n_params() - (1 if cfg.tie_embeddings and (cfg.layers is None or cfg.arch == "ledinex")
+                                                        else 2) * cfg.vocab * cfg.hidden) / L / 1e6, 1),
                               "prefill_tok_s": round(B * P / t_pre), "prefill_tokens": P,
                               "decode_tok_s": round(B * NEW / t_dec), "decode_batch": B, "decode_context": P,
                               "decode_ms_per_step": round(t_dec / NEW * 1e3, 3),

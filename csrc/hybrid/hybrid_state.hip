@@ -47,7 +47,9 @@ RT_DEVICE Tap tap_of(int k, int t, int local, int64_t pos, int taps) {
 
 // state layout: state[slot][sub][i][W], i < keep (= max(taps - 1, 1) rows), oldest first: row i of a
 // sequence whose span starts at position p0 holds the input of position p0 - (taps - 1) + i.
-template <typename OT, typename YT>
+// TAPS: the taps as a compile-time number (0: no convolution, only the add), or kMaxTaps for any
+// number up to that (`taps` at run time)
+template <typename OT, typename YT, int TAPS>
 __global__ void __launch_bounds__(kThreads) canon_add_kernel(
     OT* __restrict__ h, float* __restrict__ xs, const float* __restrict__ x, const YT* __restrict__ y,
     const YT* __restrict__ y2, const float* __restrict__ nw, float eps, const float* __restrict__ cw,
@@ -55,50 +57,58 @@ __global__ void __launch_bounds__(kThreads) canon_add_kernel(
     const int* __restrict__ start_pos, const int* __restrict__ slots, int W, int taps, int keep, int shift_state) {
   __shared__ float scratch[16];
   const int t = blockIdx.x;
-  float inv[kMaxTaps];
-  Tap tp[kMaxTaps];
+  // (loops over the taps are unrolled with a guard, so that per-tap values stay in registers)
+  constexpr int NT = TAPS == 0 ? 1 : TAPS;
+  if (TAPS != kMaxTaps) taps = TAPS;
+  float inv[NT];
   float* st = nullptr;
   int64_t pos = 0;
+  int local = 0;
   if (cw != nullptr) {
     const int s = row_seq[t];
     pos = positions[t];
-    const int local = (int)(pos - start_pos[s]);
+    local = (int)(pos - start_pos[s]);
     st = state + ((size_t)slots[s] * nsub + sub) * keep * W;
-    for (int k = 0; k < taps; ++k) tp[k] = tap_of(k, t, local, pos, taps);
   } else {
-    taps = 1;
-    tp[0].kind = 1;
-    tp[0].at = (size_t)t;
+    taps = 1;     // only the add: tap 0 is this row
   }
-  for (int k = 0; k < taps; ++k) {
+#pragma unroll
+  for (int k = 0; k < NT; ++k) {
     inv[k] = 0.f;
-    if (y != nullptr && tp[k].kind == 1) {
-      const YT* yr = y + tp[k].at * W;
-      const YT* y2r = y2 ? y2 + tp[k].at * W : nullptr;
-      float ss = 0.f;
-      for (int c = threadIdx.x; c < W; c += blockDim.x) {
-        const float v = DT<YT>::load(yr + c) + (y2r ? DT<YT>::load(y2r + c) : 0.f);
-        ss += v * v;
+    if (k < taps && y != nullptr) {
+      const Tap tp = tap_of(k, t, local, pos, taps);
+      if (tp.kind == 1) {
+        const YT* yr = y + tp.at * W;
+        const YT* y2r = y2 ? y2 + tp.at * W : nullptr;
+        float ss = 0.f;
+        for (int c = threadIdx.x; c < W; c += blockDim.x) {
+          const float v = DT<YT>::load(yr + c) + (y2r ? DT<YT>::load(y2r + c) : 0.f);
+          ss += v * v;
+        }
+        inv[k] = rsqrtf(rt::block_sum(ss, scratch) / W + eps);
       }
-      inv[k] = rsqrtf(rt::block_sum(ss, scratch) / W + eps);
     }
   }
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
     float acc = 0.f, v0 = 0.f;
     const float nwc = y != nullptr ? nw[c] : 0.f;
-    for (int k = 0; k < taps; ++k) {
-      float v = 0.f;
-      if (tp[k].kind == 1) {
-        v = x[tp[k].at * W + c];
-        if (y != nullptr) {
-          const float yy = DT<YT>::load(y + tp[k].at * W + c) + (y2 ? DT<YT>::load(y2 + tp[k].at * W + c) : 0.f);
-          v += yy * inv[k] * nwc;
+#pragma unroll
+    for (int k = 0; k < NT; ++k) {
+      if (k < taps) {
+        const Tap tp = tap_of(k, t, local, pos, taps);
+        float v = 0.f;
+        if (tp.kind == 1) {
+          v = x[tp.at * W + c];
+          if (y != nullptr) {
+            const float yy = DT<YT>::load(y + tp.at * W + c) + (y2 ? DT<YT>::load(y2 + tp.at * W + c) : 0.f);
+            v += yy * inv[k] * nwc;
+          }
+        } else if (tp.kind == 2) {
+          v = st[tp.at * W + c];
         }
-      } else if (tp[k].kind == 2) {
-        v = st[tp[k].at * W + c];
+        if (k == 0) v0 = v;
+        if (cw != nullptr) acc += cw[(size_t)c * taps + (taps - 1 - k)] * v;
       }
-      if (k == 0) v0 = v;
-      if (cw != nullptr) acc += cw[(size_t)c * taps + (taps - 1 - k)] * v;
     }
     if (y != nullptr) xs[(size_t)t * W + c] = v0;
     if (cw != nullptr) {
@@ -129,13 +139,18 @@ __global__ void __launch_bounds__(kThreads) conv_state_kernel(const XT* __restri
   const int p0 = start_pos[s];
   for (int c = threadIdx.x; c < C; c += blockDim.x) {
     float nv[kMaxTaps];
-    for (int i = 0; i < keep; ++i) {
-      const int idx = n - keep + i;   // row of this span, or (< 0) a row of the old state
-      if (idx >= 0) nv[i] = DT<XT>::load(x + (size_t)(r0 + idx) * stride + col_off + c);
-      else if (p0 + idx >= 0) nv[i] = st[(size_t)(keep + idx) * C + c];
-      else nv[i] = 0.f;
+#pragma unroll
+    for (int i = 0; i < kMaxTaps; ++i) {
+      nv[i] = 0.f;
+      if (i < keep) {
+        const int idx = n - keep + i;   // row of this span, or (< 0) a row of the old state
+        if (idx >= 0) nv[i] = DT<XT>::load(x + (size_t)(r0 + idx) * stride + col_off + c);
+        else if (p0 + idx >= 0) nv[i] = st[(size_t)(keep + idx) * C + c];
+      }
     }
-    for (int i = 0; i < keep; ++i) st[(size_t)i * C + c] = nv[i];
+#pragma unroll
+    for (int i = 0; i < kMaxTaps; ++i)
+      if (i < keep) st[(size_t)i * C + c] = nv[i];
   }
 }
 
@@ -308,14 +323,13 @@ __global__ void __launch_bounds__(kThreads) delta_prep_kernel(
   const int64_t pos = positions[t];
   const int local = (int)(pos - start_pos[s]);
   float* st = state + (size_t)slots[s] * keep * C;
-  Tap tp[kMaxTaps];
-  for (int k = 0; k < taps; ++k) tp[k] = tap_of(k, t, local, pos, taps);
   for (int c = threadIdx.x; c < C; c += blockDim.x) {
     float acc = 0.f, v0 = 0.f;
     for (int k = 0; k < taps; ++k) {
+      const Tap tp = tap_of(k, t, local, pos, taps);
       float v = 0.f;
-      if (tp[k].kind == 1) v = DT<T>::load(proj + tp[k].at * stride + q_off + c);
-      else if (tp[k].kind == 2) v = st[tp[k].at * C + c];
+      if (tp.kind == 1) v = DT<T>::load(proj + tp.at * stride + q_off + c);
+      else if (tp.kind == 2) v = st[tp.at * C + c];
       if (k == 0) v0 = v;
       acc += cw[(size_t)c * taps + (taps - 1 - k)] * v;
     }
@@ -397,16 +411,23 @@ void launch_canon_add(void* h, float* xs, const float* x, const void* y, const v
                       const int* start_pos, const int* slots, int T, int W, int taps, int keep, bool out_bf, bool y_bf,
                       bool shift_state, hipStream_t stream) {
   if (T <= 0) return;
+#define RT_CA2(OT, YT, TP)                                                                                             \
+  canon_add_kernel<OT, YT, TP><<<T, kThreads, 0, stream>>>((OT*)h, xs, x, (const YT*)y, (const YT*)y2, nw, eps, cw,     \
+                                                           state, sub, nsub, row_seq, positions, start_pos, slots, W,    \
+                                                           taps, keep, shift_state ? 1 : 0)
 #define RT_CA(OT, YT)                                                                                                  \
-  canon_add_kernel<OT, YT><<<T, kThreads, 0, stream>>>((OT*)h, xs, x, (const YT*)y, (const YT*)y2, nw, eps, cw, state, \
-                                                       sub, nsub, row_seq, positions, start_pos, slots, W, taps, keep,  \
-                                                       shift_state ? 1 : 0)
+  do {                                                                                                                 \
+    const int tp = cw == nullptr ? 0 : taps;                                                                           \
+    if (tp == 0) RT_CA2(OT, YT, 0); else if (tp == 1) RT_CA2(OT, YT, 1); else if (tp == 2) RT_CA2(OT, YT, 2);          \
+    else if (tp == 3) RT_CA2(OT, YT, 3); else if (tp == 4) RT_CA2(OT, YT, 4); else RT_CA2(OT, YT, kMaxTaps);           \
+  } while (0)
   if (out_bf) {
     if (y_bf) RT_CA(uint16_t, uint16_t); else RT_CA(uint16_t, float);
   } else {
     if (y_bf) RT_CA(float, uint16_t); else RT_CA(float, float);
   }
 #undef RT_CA
+#undef RT_CA2
 }
 
 void launch_conv_state(const void* x, int stride, int col_off, int C, float* state, int sub, int nsub, int keep,

@@ -626,7 +626,7 @@ def ledinex_config(name: str, n_layers: int, width: int, heads: int, kv_heads: i
     in turn; every feed-forward a mixture of ``experts`` squared-ReLU experts (``top`` per token,
     together ``ff`` wide unless ``expert_ff`` is given) plus a shared expert."""
     A = rec_heads or width // rec_dim
-    eff = expert_ff or max(32, ff // (top + 1))
+    eff = expert_ff or max(64, ff // (top + 1) // 64 * 64)
     mlp = {"kind": "moe", "expert": {"ff": eff}, "router": {"experts": experts, "top": top},
            "shared": {"ff": shared_ff or eff}} if ff else None
     left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5}
