@@ -50,7 +50,7 @@ RT_DEVICE Tap tap_of(int k, int t, int local, int64_t pos, int taps) {
 // TAPS: the taps as a compile-time number (0: no convolution, only the add), or kMaxTaps for any
 // number up to that (`taps` at run time)
 template <typename OT, typename YT, int TAPS>
-__global__ void __launch_bounds__(kThreads) canon_add_kernel(
+__global__ void __launch_bounds__(1024) canon_add_kernel(
     OT* __restrict__ h, float* __restrict__ xs, const float* __restrict__ x, const YT* __restrict__ y,
     const YT* __restrict__ y2, const float* __restrict__ nw, float eps, const float* __restrict__ cw,
     float* __restrict__ state, int sub, int nsub, const int* __restrict__ row_seq, const int64_t* __restrict__ positions,
@@ -309,7 +309,7 @@ __global__ void __launch_bounds__(kThreads) removal_prep_kernel(
 
 // dynamic LDS: z [C] (convolved, silu), then the unit factors of the G query heads and G key heads
 template <typename T>
-__global__ void __launch_bounds__(kThreads) delta_prep_kernel(
+__global__ void __launch_bounds__(1024) delta_prep_kernel(
     float* __restrict__ five, float* __restrict__ vout, const T* __restrict__ proj, int stride, int q_off, int b_off,
     int a_off, const float* __restrict__ cw, float* __restrict__ state, const float* __restrict__ neg_rate,
     const float* __restrict__ dt_bias, int Tn, int A, int G, int D, int E, int taps, int keep,
@@ -411,8 +411,11 @@ void launch_canon_add(void* h, float* xs, const float* x, const void* y, const v
                       const int* start_pos, const int* slots, int T, int W, int taps, int keep, bool out_bf, bool y_bf,
                       bool shift_state, hipStream_t stream) {
   if (T <= 0) return;
+  // about one entry per lane (64 .. 1024 lanes): a row's loads leave together, which is what a
+  // decode step of a few rows waits for
+  const int th = W >= 1024 ? 1024 : W <= 64 ? 64 : (W + 63) / 64 * 64;
 #define RT_CA2(OT, YT, TP)                                                                                             \
-  canon_add_kernel<OT, YT, TP><<<T, kThreads, 0, stream>>>((OT*)h, xs, x, (const YT*)y, (const YT*)y2, nw, eps, cw,     \
+  canon_add_kernel<OT, YT, TP><<<T, th, 0, stream>>>((OT*)h, xs, x, (const YT*)y, (const YT*)y2, nw, eps, cw,     \
                                                            state, sub, nsub, row_seq, positions, start_pos, slots, W,    \
                                                            taps, keep, shift_state ? 1 : 0)
 #define RT_CA(OT, YT)                                                                                                  \
@@ -503,13 +506,15 @@ int launch_delta_prep(float* five, float* vout, const void* proj, int stride, in
   if (T <= 0) return 0;
   const size_t shm = sizeof(float) * ((size_t)2 * G * D + (size_t)A * E + 2 * G);
   if (shm > 150 * 1024 || taps > kMaxTaps) return -1;
+  const int C = 2 * G * D + A * E;
+  const int th = C >= 1024 ? 1024 : C <= 256 ? 256 : (C + 63) / 64 * 64;
 #define RT_DP(TT)                                                                                                      \
   do {                                                                                                                 \
     auto kern = delta_prep_kernel<TT>;                                                                                 \
     if (shm > 48 * 1024 &&                                                                                             \
         hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm) != hipSuccess)    \
       return -2;                                                                                                       \
-    kern<<<T, kThreads, shm, stream>>>(five, vout, (const TT*)proj, stride, q_off, b_off, a_off, cw, state, neg_rate,   \
+    kern<<<T, th, shm, stream>>>(five, vout, (const TT*)proj, stride, q_off, b_off, a_off, cw, state, neg_rate,         \
                                        dt_bias, T, A, G, D, E, taps, keep, row_seq, positions, start_pos, slots,       \
                                        shift_state ? 1 : 0);                                                           \
   } while (0)
