@@ -48,6 +48,8 @@ void launch_silu_glu(void* out, const void* gu, int64_t rows, int F, bool bf, hi
 int launch_topk_softmax(int* idx, float* wt, const float* logits, int T, int E, int top, hipStream_t stream);
 int launch_moe_rows(void* out, float* hid, const void* h, const void* wgu, const void* wd, const int* idx,
                     const float* wt, int T, int W, int F, int top, int act, bool bf, hipStream_t stream);
+int launch_route_topk(int* idx, float* wt, const void* h, const float* wr, const float* bias, int T, int W, int E,
+                      int top, bool bf, hipStream_t stream);
 void launch_canon_add(void* h, float* xs, const float* x, const void* y, const void* y2, const float* nw, float eps,
                       const float* cw, float* state, int sub, int nsub, const int* row_seq, const int64_t* positions,
                       const int* start_pos, const int* slots, int T, int W, int taps, int keep, bool out_bf, bool y_bf,
@@ -376,6 +378,17 @@ void topk_softmax(torch::Tensor idx, torch::Tensor wt, torch::Tensor logits) {
 }
 
 // wgu [E, 2F, W] (gate rows, then up rows), wd [E, W, F]; idx / wt [T, top]; hid fp32 [T, top, F] scratch
+void route_topk(torch::Tensor idx, torch::Tensor wt, torch::Tensor h, torch::Tensor wr, c10::optional<torch::Tensor> bias) {
+  chk_act(h, "h"); chk_f32(wr, "router"); chk_i32(idx, "idx"); chk_f32(wt, "wt", idx.numel());
+  TORCH_CHECK(h.dim() == 2 && wr.dim() == 2 && idx.dim() == 2 && wr.size(1) == h.size(1) && idx.size(0) == h.size(0),
+              "route_topk: h [T, W], router [E, W], idx [T, top]");
+  const float* bp = nullptr;
+  if (bias.has_value()) { chk_f32(*bias, "bias", wr.size(0)); bp = bias->data_ptr<float>(); }
+  int rc = launch_route_topk(idx.data_ptr<int>(), wt.data_ptr<float>(), h.data_ptr(), wr.data_ptr<float>(), bp,
+                             (int)h.size(0), (int)h.size(1), (int)wr.size(0), (int)idx.size(1), is_bf(h), cur());
+  TORCH_CHECK(rc == 0, "route_topk: at most 512 experts, 64 choices and a row of 48 KiB (code ", rc, ")");
+}
+
 void moe_rows(torch::Tensor out, torch::Tensor hid, torch::Tensor h, torch::Tensor wgu, torch::Tensor wd, torch::Tensor idx,
               torch::Tensor wt, int64_t act) {
   chk_act(out, "out"); chk_act(h, "h"); chk_act(wgu, "wgu"); chk_act(wd, "wd"); chk_f32(hid, "hid");
@@ -657,6 +670,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("xielu", &xielu);
   m.def("silu_glu", &silu_glu);
   m.def("topk_softmax", &topk_softmax);
+  m.def("route_topk", &route_topk);
   m.def("moe_rows", &moe_rows, py::arg("out"), py::arg("hid"), py::arg("h"), py::arg("wgu"), py::arg("wd"), py::arg("idx"),
         py::arg("wt"), py::arg("act") = 0);
   m.def("limited_glu", &limited_glu);

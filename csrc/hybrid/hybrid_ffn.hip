@@ -40,14 +40,13 @@ __global__ void __launch_bounds__(256) silu_glu_kernel(T* __restrict__ out, cons
 
 constexpr int kTopPerLane = 8;      // experts per lane: up to 512 experts
 
-__global__ void __launch_bounds__(64) topk_softmax_kernel(int* __restrict__ idx, float* __restrict__ wt,
-                                                          const float* __restrict__ logits, int E, int top) {
-  const int t = blockIdx.x, lane = threadIdx.x;
+// one wave: the `top` largest of a row of E logits (lower index wins a tie) and the softmax over them
+RT_DEVICE void topk_row(int* __restrict__ idx, float* __restrict__ wt, const float* lg, int E, int top, int lane) {
   float v[kTopPerLane];
 #pragma unroll
   for (int q = 0; q < kTopPerLane; ++q) {
     const int e = lane + 64 * q;
-    v[q] = e < E ? logits[(size_t)t * E + e] : -INFINITY;
+    v[q] = e < E ? lg[e] : -INFINITY;
   }
   float mine = 0.f, first = 0.f;      // lane k keeps the k-th chosen logit
   int mine_e = 0;
@@ -75,9 +74,37 @@ __global__ void __launch_bounds__(64) topk_softmax_kernel(int* __restrict__ idx,
   const float e = lane < top ? expf(mine - first) : 0.f;
   const float sum = rt::wave_sum(e);
   if (lane < top) {
-    idx[(size_t)t * top + lane] = mine_e;
-    wt[(size_t)t * top + lane] = e / sum;
+    idx[lane] = mine_e;
+    wt[lane] = e / sum;
   }
+}
+
+__global__ void __launch_bounds__(64) topk_softmax_kernel(int* __restrict__ idx, float* __restrict__ wt,
+                                                          const float* __restrict__ logits, int E, int top) {
+  const int t = blockIdx.x;
+  topk_row(idx + (size_t)t * top, wt + (size_t)t * top, logits + (size_t)t * E, E, top, threadIdx.x);
+}
+
+// router and choice in one launch: logits = W_router h (+ bias) in fp32 from the row in LDS, one
+// wave per expert in turn, then wave 0 chooses. dynamic LDS: the row [W], the logits [E]
+template <typename T>
+__global__ void __launch_bounds__(256) route_topk_kernel(int* __restrict__ idx, float* __restrict__ wt,
+                                                         const T* __restrict__ h, const float* __restrict__ wr,
+                                                         const float* __restrict__ bias, int W, int E, int top) {
+  extern __shared__ float rl[];
+  float* lg = rl + W;
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) rl[c] = DT<T>::load(h + (size_t)t * W + c);
+  __syncthreads();
+  for (int e = wave; e < E; e += nw) {
+    const float* w = wr + (size_t)e * W;
+    float acc = 0.f;
+    for (int c = lane; c < W; c += 64) acc += w[c] * rl[c];
+    acc = rt::wave_sum(acc);
+    if (lane == 0) lg[e] = acc + (bias ? bias[e] : 0.f);
+  }
+  __syncthreads();
+  if (wave == 0) topk_row(idx + (size_t)t * top, wt + (size_t)t * top, lg, E, top, lane);
 }
 
 // R dot products at once for the whole wave: rows w, w + rs, ... (the first `ok` of them) against
@@ -247,6 +274,17 @@ int launch_topk_softmax(int* idx, float* wt, const float* logits, int T, int E, 
   if (T <= 0) return 0;
   if (E > 64 * kTopPerLane || top > 64 || top < 1 || top > E) return -1;
   topk_softmax_kernel<<<T, 64, 0, stream>>>(idx, wt, logits, E, top);
+  return 0;
+}
+
+int launch_route_topk(int* idx, float* wt, const void* h, const float* wr, const float* bias, int T, int W, int E,
+                      int top, bool bf, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (E > 64 * kTopPerLane || top > 64 || top < 1 || top > E) return -1;
+  const size_t shm = sizeof(float) * ((size_t)W + E);
+  if (shm > 48 * 1024) return -2;
+  if (bf) route_topk_kernel<uint16_t><<<T, 256, shm, stream>>>(idx, wt, (const uint16_t*)h, wr, bias, W, E, top);
+  else route_topk_kernel<float><<<T, 256, shm, stream>>>(idx, wt, (const float*)h, wr, bias, W, E, top);
   return 0;
 }
 

@@ -487,7 +487,9 @@ def test_experts_router_and_shared_expert(run, rows):
         P[f"e{e}.down"] = (torch.randn(W, F, generator=g) / F ** 0.5).to(dt).double()
     want = O.moe_ff(h.double(), P, "", {"router": {"experts": E, "top": top}})
     hd = h.to(dt).to(dev)
-    idx, wt = Hy.topk_softmax(torch.nn.functional.linear(hd.float(), P["router"].float().to(dev)), top)
+    idx, wt = Hy.route_topk(hd, P["router"].float().to(dev), top)          # one launch on the GPU
+    idx2, wt2 = Hy.topk_softmax(torch.nn.functional.linear(hd.float(), P["router"].float().to(dev)), top)
+    assert torch.equal(idx.cpu(), idx2.cpu()) and float((wt - wt2).abs().max()) < 1e-5
     up = torch.stack([P[f"e{e}.up"] for e in range(E)]).to(dt).to(dev)
     down = torch.stack([P[f"e{e}.down"] for e in range(E)]).to(dt).to(dev)
     for by_row in (None, False):

@@ -34,7 +34,7 @@ them in one batch; only the attention launch differs):
                                                 step size and decay per head
       o    = state_scan(s); pending = head_norm_gate(o) @ Wo^T
     h, x   = canon_add(x, pending)              C1, second convolution state
-    idx, wt = topk_softmax(h @ Wrouter^T)       fp32 GEMM, H11 (HIP)
+    idx, wt = route_topk(h, Wrouter)            H11 (HIP): fp32 router logits and the choice, one launch
     pending = moe_experts(h, idx, wt) (+) relu2(h @ Wsu^T) @ Wsd^T      H12 / H10, C8 (HIP)
 
 The residual stream, every norm, positions and angles, scores and softmax, the router, the
@@ -239,7 +239,7 @@ class LedinexModel(GoganexModel):
                                     b.slots, adt, shift_state=decode)
                 if not decode:
                     Hy.conv_state_update(x, 0, cfg.hidden, conv, 1, b.cu_q, b.start_pos, b.slots)
-                idx, wt = Hy.topk_softmax(F.linear(h.float(), lw["mlp.router"]), ls.moe.top)
+                idx, wt = Hy.route_topk(h, lw["mlp.router"], ls.moe.top)
                 pend = Hy.moe_experts(h, idx, wt, lw["w_up"], lw["w_down"], adt, act="relu2")
                 if ls.moe.shared_ff:
                     pend2 = self._linear(Hy.relu2(self._linear(h, l, "mlp.shared.up", skinny), adt), l, "mlp.shared.down",
