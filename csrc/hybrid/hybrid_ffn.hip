@@ -85,23 +85,55 @@ __global__ void __launch_bounds__(64) topk_softmax_kernel(int* __restrict__ idx,
   topk_row(idx + (size_t)t * top, wt + (size_t)t * top, logits + (size_t)t * E, E, top, threadIdx.x);
 }
 
-// router and choice in one launch: logits = W_router h (+ bias) in fp32 from the row in LDS, one
-// wave per expert in turn, then wave 0 chooses. dynamic LDS: the row [W], the logits [E]
+// router and choice in one launch: logits = W_router h (+ bias) in fp32 from the row in LDS — eight
+// experts at a time, every lane's weight loads of a batch in flight together (16-byte loads when the
+// row allows), wave sums, partials through LDS — then wave 0 chooses.
+// dynamic LDS: the row [W], the logits [E], the partials [E][waves]
+constexpr int kRouteBatch = 8;
 template <typename T>
 __global__ void __launch_bounds__(256) route_topk_kernel(int* __restrict__ idx, float* __restrict__ wt,
                                                          const T* __restrict__ h, const float* __restrict__ wr,
-                                                         const float* __restrict__ bias, int W, int E, int top) {
-  extern __shared__ float rl[];
-  float* lg = rl + W;
+                                                         const float* __restrict__ bias, int W, int E, int top, int vec) {
+  extern __shared__ float4 rl4[];       // (16-byte aligned: the row is read in 16-byte pieces)
+  float* rl = reinterpret_cast<float*>(rl4);
+  const int Wp = (W + 3) & ~3;
+  float* lg = rl + Wp;
+  float* part = lg + E;
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   for (int c = threadIdx.x; c < W; c += blockDim.x) rl[c] = DT<T>::load(h + (size_t)t * W + c);
   __syncthreads();
-  for (int e = wave; e < E; e += nw) {
-    const float* w = wr + (size_t)e * W;
-    float acc = 0.f;
-    for (int c = lane; c < W; c += 64) acc += w[c] * rl[c];
-    acc = rt::wave_sum(acc);
-    if (lane == 0) lg[e] = acc + (bias ? bias[e] : 0.f);
+  for (int e0 = 0; e0 < E; e0 += kRouteBatch) {
+    float acc[kRouteBatch];
+#pragma unroll
+    for (int j = 0; j < kRouteBatch; ++j) acc[j] = 0.f;
+    if (vec) {
+      for (int c = threadIdx.x * 4; c < W; c += blockDim.x * 4) {
+        const float4 x = *reinterpret_cast<const float4*>(rl + c);
+        float4 w4[kRouteBatch];
+#pragma unroll
+        for (int j = 0; j < kRouteBatch; ++j)
+          w4[j] = *reinterpret_cast<const float4*>(wr + (size_t)min(e0 + j, E - 1) * W + c);
+#pragma unroll
+        for (int j = 0; j < kRouteBatch; ++j) acc[j] += w4[j].x * x.x + w4[j].y * x.y + w4[j].z * x.z + w4[j].w * x.w;
+      }
+    } else {
+      for (int c = threadIdx.x; c < W; c += blockDim.x) {
+        const float x = rl[c];
+#pragma unroll
+        for (int j = 0; j < kRouteBatch; ++j) acc[j] += wr[(size_t)min(e0 + j, E - 1) * W + c] * x;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kRouteBatch; ++j) {
+      const float v = rt::wave_sum(acc[j]);
+      if (lane == 0 && e0 + j < E) part[(e0 + j) * nw + wave] = v;
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += blockDim.x) {
+    float v = bias ? bias[e] : 0.f;
+    for (int w = 0; w < nw; ++w) v += part[e * nw + w];
+    lg[e] = v;
   }
   __syncthreads();
   if (wave == 0) topk_row(idx + (size_t)t * top, wt + (size_t)t * top, lg, E, top, lane);
@@ -281,10 +313,11 @@ int launch_route_topk(int* idx, float* wt, const void* h, const float* wr, const
                       int top, bool bf, hipStream_t stream) {
   if (T <= 0) return 0;
   if (E > 64 * kTopPerLane || top > 64 || top < 1 || top > E) return -1;
-  const size_t shm = sizeof(float) * ((size_t)W + E);
+  const size_t shm = sizeof(float) * ((size_t)((W + 3) & ~3) + 5 * (size_t)E);
   if (shm > 48 * 1024) return -2;
-  if (bf) route_topk_kernel<uint16_t><<<T, 256, shm, stream>>>(idx, wt, (const uint16_t*)h, wr, bias, W, E, top);
-  else route_topk_kernel<float><<<T, 256, shm, stream>>>(idx, wt, (const float*)h, wr, bias, W, E, top);
+  const int vec = (W & 3) == 0 && (reinterpret_cast<uintptr_t>(wr) & 15) == 0 ? 1 : 0;
+  if (bf) route_topk_kernel<uint16_t><<<T, 256, shm, stream>>>(idx, wt, (const uint16_t*)h, wr, bias, W, E, top, vec);
+  else route_topk_kernel<float><<<T, 256, shm, stream>>>(idx, wt, (const float*)h, wr, bias, W, E, top, vec);
   return 0;
 }
 

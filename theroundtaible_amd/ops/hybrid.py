@@ -354,7 +354,7 @@ def route_topk(h, router_w, top: int, bias=None) -> Tuple[torch.Tensor, torch.Te
     """Router and choice: fp32 logits ``router_w`` [E, W] . ``h`` [T, W] (+ ``bias``), then as
     :func:`topk_softmax`. One launch on the GPU (the row in LDS, a wave per expert in turn)."""
     E, W = router_w.shape
-    if _gpu(h) and E <= 512 and top <= 64 and (W + E) * 4 <= 48 * 1024:
+    if _gpu(h) and E <= 512 and top <= 64 and (W + 4 + 5 * E) * 4 <= 48 * 1024:
         idx = torch.empty(h.shape[0], top, dtype=torch.int32, device=h.device)
         wt = torch.empty(h.shape[0], top, dtype=torch.float32, device=h.device)
         native().route_topk(idx, wt, h.contiguous(), router_w, bias)
