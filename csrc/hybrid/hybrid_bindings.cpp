@@ -77,7 +77,7 @@ void launch_head_norm_gate(void* out, int out_stride, int out_off, const float* 
                            bool out_bf, bool gate_bf, hipStream_t stream);
 int launch_state_scan(float* out, const float* q, const float* k, const float* v, const float* w, const float* a,
                       const float* b, int sq, int sk, int sv, int sw, int sa, int sb, const float* decay, float* state,
-                      const int* cu_q, const int* start_pos, const int* slots, int S, int A, int D, int E,
+                      const int* cu_q, const int* start_pos, const int* slots, int S, int T, int A, int D, int E,
                       hipStream_t stream);
 
 namespace {
@@ -620,7 +620,7 @@ void state_scan(torch::Tensor out, torch::Tensor q, torch::Tensor k, torch::Tens
   chk_i32(cu_q, "cu_q"); chk_i32(start_pos, "start_pos", S); chk_i32(slots, "slots", S);
   int rc = launch_state_scan(out.data_ptr<float>(), qp, kp, vp, wp, ap, bp, sq, sk, sv, sw, sa, sb,
                              opt_f32(decay, "decay", A), state.data_ptr<float>(), cu_q.data_ptr<int>(),
-                             start_pos.data_ptr<int>(), slots.data_ptr<int>(), (int)S, (int)A, (int)D, (int)E, cur());
+                             start_pos.data_ptr<int>(), slots.data_ptr<int>(), (int)S, (int)T, (int)A, (int)D, (int)E, cur());
   TORCH_CHECK(rc == 0, "state_scan: unsupported shape (code ", rc, ")");
 }
 

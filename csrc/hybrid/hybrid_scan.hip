@@ -13,7 +13,9 @@
 // 4 rows per lane: about 20 FMAs and 8 DPP adds per token. One workgroup of 256 lanes =
 // (sequence, head, 256 / P columns). Tokens are staged through LDS in chunks of 16: the next
 // chunk's streams are loaded into registers (16-byte loads) while the current chunk is computed,
-// and the chunk's outputs leave through LDS so that global writes are whole lines. The state is
+// the operands of the next token are read from LDS while the current one is computed (a whole chunk
+// is unrolled over two operand sets), and a lane's share of q . S goes to LDS as it is: the shares
+// of a column are added when the chunk's outputs are written, as whole lines. The state is
 // kept column by column, [slot][head][E][D], so that a lane's rows are contiguous.
 #include "../common.h"
 
@@ -47,7 +49,9 @@ RT_DEVICE float4 load4(const float* __restrict__ row, int r, int D, bool vec) {
   return o;
 }
 
-template <int DR, bool HAS_W, bool HAS_AB>
+// UNROLL: whole chunks run unrolled (prompts); without it the code is a fraction of the size, which is
+// what a launch over single rows (a decode step, cold instruction cache) is timed by
+template <int DR, bool HAS_W, bool HAS_AB, bool UNROLL>
 __global__ void __launch_bounds__(kScanThreads) state_scan_kernel(
     float* __restrict__ out, const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
     const float* __restrict__ w, const float* __restrict__ a, const float* __restrict__ b, int sq, int sk, int sv, int sw,
@@ -67,7 +71,7 @@ __global__ void __launch_bounds__(kScanThreads) state_scan_kernel(
   if (n <= 0) return;
   float4* str = lds4;                                             // [kTT][NS][Dp4]
   float* vs = reinterpret_cast<float*>(str + kTT * NS * Dp4);     // [kTT][CB]
-  float* os = vs + kTT * CB;                                      // [kTT][CB]
+  float* os = vs + kTT * CB;                                      // [kTT][256]: every lane's share of q . S
   const int row_lo = part * DR;
   const bool live = col < E;
   float S[DR];
@@ -135,9 +139,42 @@ __global__ void __launch_bounds__(kScanThreads) state_scan_kernel(
       if (l < nv) vs[threadIdx.x + l * kScanThreads] = prev[l];
     __syncthreads();
     if (c0 + kTT < n) fetch(c0 + kTT);      // in flight while this chunk is computed
-    // the operands of token tok + 1 are read from LDS while token tok is computed
-    float4 cq[R4], ck[R4], cw[R4], ca[R4], cb[R4], nq[R4], nk[R4], nw[R4], na[R4], nb[R4];
-    float cv, nvv;
+    // One token: s = b . S (summed over the column's lanes, the only cross-lane step on the chain),
+    // the update, and this lane's share of q . S, which goes to LDS as it is: the shares of a
+    // column are added when the chunk's outputs are written, not inside the token loop.
+    auto step = [&](int tok, const float4* tq, const float4* tk, const float4* tw, const float4* ta, const float4* tb,
+                    float vv) {
+      float sv_ = 0.f;
+      if (HAS_AB) {
+#pragma unroll
+        for (int i4 = 0; i4 < R4; ++i4) {
+          const float4 bb = tb[i4];
+          sv_ += bb.x * S[i4 * 4] + bb.y * S[i4 * 4 + 1] + bb.z * S[i4 * 4 + 2] + bb.w * S[i4 * 4 + 3];
+        }
+        sv_ = group_sum(sv_, P);
+      }
+      float acc = 0.f;
+#pragma unroll
+      for (int i4 = 0; i4 < R4; ++i4) {
+        const float4 kk = tk[i4], qq = tq[i4];
+        float u0 = kk.x * vv, u1 = kk.y * vv, u2 = kk.z * vv, u3 = kk.w * vv;
+        if (HAS_AB) {
+          const float4 aa = ta[i4];
+          u0 -= aa.x * sv_; u1 -= aa.y * sv_; u2 -= aa.z * sv_; u3 -= aa.w * sv_;
+        }
+        float d0 = dconst, d1 = dconst, d2 = dconst, d3 = dconst;
+        if (HAS_W) {
+          const float4 ww = tw[i4];
+          d0 = ww.x; d1 = ww.y; d2 = ww.z; d3 = ww.w;
+        }
+        S[i4 * 4] = S[i4 * 4] * d0 + u0;
+        S[i4 * 4 + 1] = S[i4 * 4 + 1] * d1 + u1;
+        S[i4 * 4 + 2] = S[i4 * 4 + 2] * d2 + u2;
+        S[i4 * 4 + 3] = S[i4 * 4 + 3] * d3 + u3;
+        acc += qq.x * S[i4 * 4] + qq.y * S[i4 * 4 + 1] + qq.z * S[i4 * 4 + 2] + qq.w * S[i4 * 4 + 3];
+      }
+      os[tok * kScanThreads + threadIdx.x] = acc;
+    };
     auto read_tok = [&](int tok, float4* tq, float4* tk, float4* tw, float4* ta, float4* tb, float& tv) {
       const float4* qs = str + (tok * NS) * Dp4 + part * R4;
       const float4* ks = qs + Dp4;
@@ -156,58 +193,34 @@ __global__ void __launch_bounds__(kScanThreads) state_scan_kernel(
       }
       tv = vs[tok * CB + cl];
     };
-    read_tok(0, cq, ck, cw, ca, cb, cv);
-    for (int tok = 0; tok < nt; ++tok) {
-      read_tok(tok + 1 < nt ? tok + 1 : tok, nq, nk, nw, na, nb, nvv);
-      const float vv = cv;
-      float sv_ = 0.f;
-      if (HAS_AB) {
+    if (UNROLL && nt == kTT) {
+      // a whole chunk: unrolled, two operand sets in turn, so the operands of token tok + 1 are
+      // read from LDS while token tok is computed and nothing is copied
+      float4 oq[2][R4], ok[2][R4], ow[2][R4], oa[2][R4], ob[2][R4];
+      float ov[2];
+      read_tok(0, oq[0], ok[0], ow[0], oa[0], ob[0], ov[0]);
 #pragma unroll
-        for (int i4 = 0; i4 < R4; ++i4) {
-          const float4 bb = cb[i4];
-          sv_ += bb.x * S[i4 * 4] + bb.y * S[i4 * 4 + 1] + bb.z * S[i4 * 4 + 2] + bb.w * S[i4 * 4 + 3];
-        }
-        sv_ = group_sum(sv_, P);
+      for (int tok = 0; tok < kTT; ++tok) {
+        const int c = tok & 1, nx = c ^ 1;
+        if (tok + 1 < kTT) read_tok(tok + 1, oq[nx], ok[nx], ow[nx], oa[nx], ob[nx], ov[nx]);
+        step(tok, oq[c], ok[c], ow[c], oa[c], ob[c], ov[c]);
       }
-      float acc = 0.f;
-#pragma unroll
-      for (int i4 = 0; i4 < R4; ++i4) {
-        const float4 kk = ck[i4], qq = cq[i4];
-        float u0 = kk.x * vv, u1 = kk.y * vv, u2 = kk.z * vv, u3 = kk.w * vv;
-        if (HAS_AB) {
-          const float4 aa = ca[i4];
-          u0 -= aa.x * sv_; u1 -= aa.y * sv_; u2 -= aa.z * sv_; u3 -= aa.w * sv_;
-        }
-        float d0 = dconst, d1 = dconst, d2 = dconst, d3 = dconst;
-        if (HAS_W) {
-          const float4 ww = cw[i4];
-          d0 = ww.x; d1 = ww.y; d2 = ww.z; d3 = ww.w;
-        }
-        S[i4 * 4] = S[i4 * 4] * d0 + u0;
-        S[i4 * 4 + 1] = S[i4 * 4 + 1] * d1 + u1;
-        S[i4 * 4 + 2] = S[i4 * 4 + 2] * d2 + u2;
-        S[i4 * 4 + 3] = S[i4 * 4 + 3] * d3 + u3;
-        acc += qq.x * S[i4 * 4] + qq.y * S[i4 * 4 + 1] + qq.z * S[i4 * 4 + 2] + qq.w * S[i4 * 4 + 3];
+    } else {
+      float4 tq[R4], tk[R4], tw[R4], ta[R4], tb[R4];
+      float tv;
+      for (int tok = 0; tok < nt; ++tok) {
+        read_tok(tok, tq, tk, tw, ta, tb, tv);
+        step(tok, tq, tk, tw, ta, tb, tv);
       }
-      acc = group_sum(acc, P);
-      if (part == 0) os[tok * CB + cl] = acc;
-#pragma unroll
-      for (int i4 = 0; i4 < R4; ++i4) {
-        cq[i4] = nq[i4];
-        ck[i4] = nk[i4];
-        if (HAS_W) cw[i4] = nw[i4];
-        if (HAS_AB) {
-          ca[i4] = na[i4];
-          cb[i4] = nb[i4];
-        }
-      }
-      cv = nvv;
     }
     __syncthreads();
     for (int i = threadIdx.x; i < nt * CB; i += kScanThreads) {
       const int tok = i / CB, c = i - tok * CB;
       const int gc = blockIdx.z * CB + c;
-      if (gc < E) out[(size_t)(r0 + c0 + tok) * A * E + head * E + gc] = os[i];
+      const float* sh = os + tok * kScanThreads + c * P;      // the column's P shares
+      float o = 0.f;
+      for (int j = 0; j < P; ++j) o += sh[j];
+      if (gc < E) out[(size_t)(r0 + c0 + tok) * A * E + head * E + gc] = o;
     }
   }
   if (live) {
@@ -240,9 +253,10 @@ static void scan_shape(int D, int& DR, int& P, int& lgP) {
 
 int launch_state_scan(float* out, const float* q, const float* k, const float* v, const float* w, const float* a,
                       const float* b, int sq, int sk, int sv, int sw, int sa, int sb, const float* decay, float* state,
-                      const int* cu_q, const int* start_pos, const int* slots, int S, int A, int D, int E,
+                      const int* cu_q, const int* start_pos, const int* slots, int S, int T, int A, int D, int E,
                       hipStream_t stream) {
   if (S <= 0) return 0;
+  const bool unroll = T > 2 * S;      // rows per span on average: single rows take the small kernel
   int DR, P, lgP;
   scan_shape(D, DR, P, lgP);
   if (P > 16 || D < 1 || E < 1) return -1;
@@ -254,11 +268,15 @@ int launch_state_scan(float* out, const float* q, const float* k, const float* v
   // 16-byte loads of the streams: every row start and the head offset on a 16-byte boundary
   auto al = [&](const float* p, int st) { return p == nullptr || ((reinterpret_cast<uintptr_t>(p) & 15) == 0 && (st & 3) == 0); };
   const int vec = (D & 3) == 0 && al(q, sq) && al(k, sk) && al(w, sw) && al(a, sa) && al(b, sb) ? 1 : 0;
-  const size_t shm = sizeof(float) * (size_t)kTT * ((size_t)NS * Dp + 2 * CB);
+  const size_t shm = sizeof(float) * (size_t)kTT * ((size_t)NS * Dp + CB + kScanThreads);
   dim3 grid(S, A, (E + CB - 1) / CB);
 #define RT_SCAN(DRV, HW, HAB)                                                                                          \
   do {                                                                                                                 \
-    auto kern = state_scan_kernel<DRV, HW, HAB>;                                                                       \
+    if (unroll) RT_SCAN_U(DRV, HW, HAB, true); else RT_SCAN_U(DRV, HW, HAB, false);                                    \
+  } while (0)
+#define RT_SCAN_U(DRV, HW, HAB, UN)                                                                                    \
+  do {                                                                                                                 \
+    auto kern = state_scan_kernel<DRV, HW, HAB, UN>;                                                                   \
     if (shm > 48 * 1024 &&                                                                                             \
         hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm) != hipSuccess)    \
       return -3;                                                                                                       \
@@ -274,5 +292,6 @@ int launch_state_scan(float* out, const float* q, const float* k, const float* v
   else RT_SCAN_DR(true, false);
 #undef RT_SCAN_DR
 #undef RT_SCAN
+#undef RT_SCAN_U
   return 0;
 }
