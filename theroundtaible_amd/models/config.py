@@ -621,7 +621,7 @@ def parse_ledinex(d: dict, name: str = "ledinex") -> ModelConfig:
 def ledinex_config(name: str, n_layers: int, width: int, heads: int, kv_heads: int, dim: int, ff: int, vocab: int,
                    pattern: Tuple[str, ...] = ("parallel_2", "delta", "parallel"), rec_heads: int = 0, rec_dim: int = 64,
                    window: int = 1024, experts: int = 8, top: int = 2, expert_ff: int = 0, shared_ff: int = 0,
-                   taps: int = 3, conv: int = 4, decay_rank: int = 64, max_pos: int = 1 << 17) -> ModelConfig:
+                   taps: int = 4, conv: int = 4, decay_rank: int = 64, max_pos: int = 1 << 17) -> ModelConfig:
     """A Ledinex stack from a few sizes (benchmarks and presets): the mixer types of ``pattern``
     in turn; every feed-forward a mixture of ``experts`` squared-ReLU experts (``top`` per token,
     together ``ff`` wide unless ``expert_ff`` is given) plus a shared expert."""
@@ -631,13 +631,13 @@ def ledinex_config(name: str, n_layers: int, width: int, heads: int, kv_heads: i
            "shared": {"ff": shared_ff or eff}} if ff else None
     left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5}
     kinds = {
-        "parallel": {"left": dict(left, softcap=30.0, rot={"base": 500000.0, "dims": dim, "scaling": {"factor": 4.0}}),
+        "parallel": {"left": dict(left, softcap=30.0, rot={"base": 500000.0, "dims": dim, "scaling": {"factor": 2.0}}),
                      "left_scale": 0.7, "right_scale": 0.7,
                      "right": {"heads": A, "dim": rec_dim, "vdim": rec_dim,
                                "decay": [math.exp(-2.0 ** (-1 - 5.0 * a / max(1, A - 1))) for a in range(A)]}},
         "parallel_2": {"left": dict(left, mask={"size": window},
-                                    rot={"base": 50000.0, "dims": dim // 2,
-                                         "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}),
+                                    rot={"base": 100000.0, "dims": dim // 2,
+                                         "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}),
                        "left_scale": 0.7, "right_scale": 0.7,
                        "right": {"heads": A, "dim": rec_dim, "decay_rank": decay_rank}},
         "delta": {"heads": A, "kv_heads": max(1, A // 2), "dim": rec_dim, "vdim": rec_dim, "conv": conv},

@@ -381,7 +381,8 @@ def moe_experts(h, idx, wt, w_gu, w_down, out_dtype, by_row: Optional[bool] = No
     the experts are W_down[e] relu(W_up[e] h)^2 and ``w_gu`` is [E, F, W]. Two forms: row by row
     (GPU steps of a few rows: two launches, no host round trip, so a captured decode step can hold
     them) and expert by expert (the rows of each expert gathered for library GEMMs, one host read of
-    the expert counts; rows are added to the fp32 sum in expert order whatever else is in the batch)."""
+    the expert counts; a row's experts are added in fp32 in the order of its choices whatever else is
+    in the batch)."""
     T, top = idx.shape
     if by_row is None:
         by_row = _gpu(h) and T <= MOE_ROWS
@@ -390,21 +391,24 @@ def moe_experts(h, idx, wt, w_gu, w_down, out_dtype, by_row: Optional[bool] = No
         hid = torch.empty(T * top * w_down.shape[2], dtype=torch.float32, device=h.device)
         native().moe_rows(out, hid, h.contiguous(), w_gu, w_down, idx, wt, 1 if act == "relu2" else 0)
         return out
-    E = w_gu.shape[0]
+    E, W = w_gu.shape[0], h.shape[1]
     flat = idx.reshape(-1).long()
-    order = torch.argsort(flat, stable=True)
+    order = torch.argsort(flat, stable=True)            # (row, choice) pairs, expert by expert
     counts = torch.bincount(flat, minlength=E).tolist()
-    rows, cw = order // top, wt.reshape(-1)[order]
-    out = torch.zeros(h.shape, dtype=torch.float32, device=h.device)
+    hs = h.index_select(0, order // top)                # every expert's input rows, gathered once
+    ys = torch.empty(T * top, W, dtype=h.dtype, device=h.device)
     at = 0
     for e, n in enumerate(counts):
         if n:
-            r = rows[at:at + n]
-            a = torch.nn.functional.linear(h.index_select(0, r), w_gu[e])
+            a = torch.nn.functional.linear(hs[at:at + n], w_gu[e])
             a = relu2(a, h.dtype) if act == "relu2" else silu_glu(a, h.dtype)
-            out.index_add_(0, r, torch.nn.functional.linear(a, w_down[e]).float() * cw[at:at + n, None])
+            torch.mm(a, w_down[e].t(), out=ys[at:at + n])
             at += n
-    return out.to(out_dtype)
+    back = torch.empty_like(order)
+    back[order] = torch.arange(T * top, device=h.device)
+    y = ys.index_select(0, back).view(T, top, W).float()
+    # a row's experts are added in the order of its choices, in fp32, whatever else is in the batch
+    return torch.bmm(wt.view(T, 1, top), y).view(T, W).to(out_dtype)
 
 
 # ---- the PyTorch statements (CPU tensors; what the kernels are tested against) ---------------------
