@@ -583,8 +583,10 @@ def parse_ledinex(d: dict, name: str = "ledinex") -> ModelConfig:
         elif kind in ("parallel", "parallel_2"):
             left, rx = _ledinex_attention(mx["left"], kind, where), mx["right"]
             if kind == "parallel":
-                right = DecaySumSpec(int(rx["heads"]), int(rx["dim"]), int(rx.get("vdim", rx["dim"])),
-                                     tuple(float(v) for v in rx["decay"]))
+                dec = rx["decay"]
+                dec = [dec] * int(rx["heads"]) if isinstance(dec, (int, float)) else dec     # one number: every head's
+                right = DecaySumSpec(int(rx["heads"]), int(rx["dim"]), int(rx.get("vdim") or rx["dim"]),
+                                     tuple(float(v) for v in dec))
                 if len(right.decay) != right.heads:
                     raise ValueError(f"{where}: {len(right.decay)} decays for {right.heads} heads")
             else:
